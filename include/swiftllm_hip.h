@@ -492,7 +492,8 @@ int swl_decode_engine_step(void *resid_out, const void *w_stream, const void *no
 
 /* ---- fp32 residual stream: embedding with learned positions, LayerNorm, fused sandwich-norm step ------------------
  * (no counterpart in the reference, which serves LLaMA only; used by the Kekapel model.) dtype may be SWL_F32.
- * swl_embed_pos:     x[t] = embed[tokens[t]] * scale + pos[positions[t]] in fp32; x0 (may be NULL) gets a copy.
+ * swl_embed_pos:     x[t] = embed[tokens[t]] * scale + pos[positions[t]] in fp32; x0 (may be NULL) gets a copy; pos NULL:
+ *                    a model without learned positions (x[t] = embed[tokens[t]] * scale).
  * swl_layernorm:     out[r] = (x[i] - mean) / sqrt(var + eps) * w + b of row i = row_idx ? row_idx[r] : r (fp32 stats,
  *                    var = mean of squared deviations); out in dtype, x / w / b fp32.
  * swl_add_layernorm: x += mult * LN(y; w1, b1) (if y) + x0 (if x0) + step (if step, a [width] vector);
@@ -542,6 +543,63 @@ int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const v
                           int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window,
                           float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
                           int32_t key_splits, float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream);
+
+/* ---- the same attention loops with the masks and denominators of other designs --------------------------------------------
+ * swl_masked_attn / swl_masked_attn_tiles are swl_window_attn / swl_window_attn_tiles with
+ *   mask_kind     0: sliding window (keys [p - window + 1, p]); 1: chunks (keys [floor(p / window) * window, p], chunks
+ *                 counted from position 0). window 0: every earlier key, whatever the kind.
+ *   sink          NULL, or fp32 [num_q_heads]: a logit per head that is added to the softmax denominator only.
+ *   num_v_heads   value heads in a page (divides num_kv_heads); key head g reads value head g % num_v_heads. Several score
+ *                 maps over the same values: lay the maps out map-major, [map][head].
+ *   out_f32       1: out is fp32 whatever dtype says of the operands.
+ *   heads_per_group (tiles only; 0: all) heads handled by one workgroup when the heads are not mixed: the heads of a tile
+ *                 are shared out over ceil(H / heads_per_group) workgroups.
+ * The tiles form serves more (dim, vdim) pairs without a mixing matrix than with one: ask swl_masked_attn_tiles_supported. */
+int swl_masked_attn(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                    const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, const float *rel, int32_t rel_len,
+                    int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim,
+                    int64_t q_tok_stride, int32_t window, float scale, float softcap, int32_t max_blocks_per_seq,
+                    int64_t block_stride, int32_t mask_kind, const float *sink, int32_t num_v_heads, int32_t out_f32,
+                    int32_t dtype, swl_stream_t stream);
+int swl_masked_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t num_v_heads, int32_t dim,
+                                    int32_t vdim, int32_t dtype);
+int swl_masked_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                          const int32_t *tok_seq, const int32_t *tok_pos, const int32_t *tile_row0,
+                          const int32_t *tile_cnt, const float *talk, const float *rel, int32_t rel_len, int32_t num_tiles,
+                          int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride,
+                          int32_t window, float scale, float softcap, int32_t max_blocks_per_seq, int64_t block_stride,
+                          int32_t key_splits, float *scratch, int64_t num_tokens, int32_t mask_kind, const float *sink,
+                          int32_t num_v_heads, int32_t out_f32, int32_t heads_per_group, int32_t dtype,
+                          swl_stream_t stream);
+
+/* ---- rotary positions on interleaved pairs fused with the paged KV store; gated / combined heads ---------------------------
+ * Rotation: dimension 2i of a head is paired with 2i + 1, i < rot_dims / 2; (u, v) at position p becomes
+ * (u cos a - v sin a, v cos a + u sin a), a = p * freq[i] (freq: float64 [rot_dims / 2] on the device; angles are evaluated
+ * in float64). dtype may be SWL_F32. Pages: keys [heads, 16, dim], values transposed [heads, vdim, 16].
+ * swl_rope_store_kv: rows [q: num_q_heads x dim | k: num_k_heads x dim | v: num_v_heads x vdim]; q rotated in place, k
+ *   rotated into the K pool, v into the V pool. k_cache NULL: queries only.
+ * swl_latent_rope_store_kv: rows hold num_heads query heads [dim | rot_dim] and, at column dkv_col (< 0: none), the
+ *   compressed row [kv_rank | rot_dim]. qa[t][h][kv_rank : kv_rank + rot_dim] = rotated query part; the RMS-normed latent
+ *   (weight c_norm, eps) and the rotated shared key part are stored as one key head of kv_rank + rot_dim and the latent
+ *   again, transposed, as one value head of kv_rank.
+ * swl_diff_head_combine: maps fp32 [T, 2, H, vdim] -> out[T, H, vdim] = unit_rms(a1 - lambda a2; eps) * mult *
+ *   sigmoid(gate[t * gate_stride + h]) (gate NULL: no gate).
+ * swl_head_gate: y[T, H, vdim] *= sigmoid(gate[t * gate_stride + h]) in place. */
+int swl_rope_store_kv(void *qkv, const double *freq, void *k_cache, void *v_cache, const int32_t *block_table,
+                      const int32_t *tok_seq, const int32_t *tok_pos, int64_t num_tokens, int32_t num_q_heads,
+                      int32_t num_k_heads, int32_t num_v_heads, int32_t dim, int32_t vdim, int32_t rot_dims,
+                      int64_t tok_stride, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                      swl_stream_t stream);
+int swl_latent_rope_store_kv(const void *proj, void *qa, const double *freq, const float *c_norm, void *k_cache,
+                             void *v_cache, const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                             int64_t num_tokens, int32_t num_heads, int32_t dim, int32_t rot_dim, int32_t kv_rank,
+                             int64_t proj_stride, int64_t dkv_col, int64_t qa_stride, int32_t max_blocks_per_seq,
+                             int64_t block_stride, float eps, int32_t dtype, swl_stream_t stream);
+int swl_diff_head_combine(void *out, const float *maps, const void *gate, int64_t gate_stride, float lambda, float mult,
+                          float eps, int64_t num_tokens, int32_t num_heads, int32_t vdim, int32_t dtype,
+                          swl_stream_t stream);
+int swl_head_gate(void *y, const void *gate, int64_t gate_stride, int64_t num_tokens, int32_t num_heads, int32_t vdim,
+                  int32_t dtype, swl_stream_t stream);
 
 /* ---- PolyNorm activation: out = a N(z) + b N(z^2) + c N(z^3) + e, N(v) = v / sqrt(mean(v^2) + eps) over the row ---------- */
 int swl_polynorm(void *out, const void *z, float a, float b, float c, float e, float eps, int64_t num_rows, int32_t ff,

@@ -102,6 +102,15 @@ SIGNATURES = {
                         _I64, _I32, _P],
     "swl_window_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32,
                               _I32, _I64, _I32, _P, _I64, _I32, _P],
+    "swl_masked_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _F32, _I32,
+                        _I64, _I32, _P, _I32, _I32, _I32, _P],
+    "swl_masked_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _F32,
+                              _F32, _I32, _I64, _I32, _P, _I64, _I32, _P, _I32, _I32, _I32, _I32, _P],
+    "swl_rope_store_kv": [_P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _I32, _I64, _I32, _P],
+    "swl_latent_rope_store_kv": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I64, _I64, _I32,
+                                 _I64, _F32, _I32, _P],
+    "swl_diff_head_combine": [_P, _P, _P, _I64, _F32, _F32, _F32, _I64, _I32, _I32, _I32, _P],
+    "swl_head_gate": [_P, _P, _I64, _I64, _I32, _I32, _I32, _P],
     "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
     "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
     "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
@@ -137,6 +146,7 @@ _SPECIAL = {
     "swl_gemm_rows_supported": ([_I32, _I32, _I32], _I32),
     "swl_moe_expert_stationary_supported": ([_I64, _I32, _I32, _I32, _I32], _I32),
     "swl_window_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32], _I32),
+    "swl_masked_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_supported": ([_I32, _I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_slots_per_layer": ([_I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_workspace_bytes": ([_I32, _I32, _I32, _I32], ctypes.c_size_t),

@@ -35,16 +35,16 @@ __device__ __forceinline__ void row_stats(const float *row, int n, float eps, fl
     rstd = 1.0f / sqrtf(var + eps);
 }
 
-// x[t] = embed[token[t]] * scale + pos[position[t]]  (fp32); x0 (optional) receives a copy.
+// x[t] = embed[token[t]] * scale + pos[position[t]]  (fp32); x0 (optional) receives a copy. pos NULL: no learned positions.
 template <typename T>
 __global__ __launch_bounds__(kLnThreads) void embed_pos_kernel(float *x, float *x0, const T *embed, const T *pos,
                                                                const int32_t *tokens, const int32_t *positions,
                                                                float scale, int width) {
     const int64_t t = blockIdx.x;
     const T *e = embed + static_cast<int64_t>(tokens[t]) * width;
-    const T *p = pos + static_cast<int64_t>(positions[t]) * width;
+    const T *p = pos ? pos + static_cast<int64_t>(positions[t]) * width : nullptr;
     for (int i = threadIdx.x; i < width; i += kLnThreads) {
-        const float v = to_f(e[i]) * scale + to_f(p[i]);
+        const float v = p ? to_f(e[i]) * scale + to_f(p[i]) : to_f(e[i]) * scale;
         x[t * width + i] = v;
         if (x0) x0[t * width + i] = v;
     }
@@ -108,7 +108,7 @@ extern "C" int swl_embed_pos(float *x, float *x0, const void *embed, const void 
                              swl_stream_t stream) {
     if (num_tokens < 0 || width <= 0) return SWL_ERR_BAD_ARG;
     if (num_tokens == 0) return SWL_OK;
-    if (!x || !embed || !pos || !tokens || !positions) return SWL_ERR_BAD_ARG;
+    if (!x || !embed || !tokens || (pos && !positions)) return SWL_ERR_BAD_ARG;
     if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
     SWL_DISPATCH_DTYPE3(dtype, T, {
         hipLaunchKernelGGL((swl::embed_pos_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kLnThreads), 0,

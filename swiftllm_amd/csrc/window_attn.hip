@@ -12,6 +12,13 @@
 //   2. mixed scores  m[h][j] = sum_g talk[h][g] s[g][j], online softmax per mixed head h (fp32, full-precision exp),
 //   3. acc[h][:] = acc[h][:] * alpha[h] + sum_j p[h][j] v[kv(h)][j][:]   (fp32 weights, fp32 accumulation).
 // This is the reference-grade kernel: everything after the loads is fp32 whatever the storage dtype.
+//
+// The general entry point (swl_masked_attn) adds what other designs need of the same loop:
+//   * mask_kind 1: chunked visibility — keys [floor(p / window) * window, p], chunks counted from position 0;
+//   * sink[H]: a learned logit per head that joins the softmax denominator only (no key, no value, not scaled);
+//   * num_v_heads < num_kv_heads: several key heads share one value head (value head = key head % num_v_heads) — two
+//     score maps over the same values, laid out map-major, are 2 G key heads over G value heads;
+//   * out_f32: the result leaves in fp32 (for a combination of maps that cancels).
 #include "swl_common.h"
 
 namespace swl {
@@ -32,14 +39,14 @@ template <typename T>
 __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const float *talk, const float *rel, int rel_len, int H, int G, int d, int dv,
-    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride) {
+    int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
+    int mask_kind, const float *sink, int GV, int out_f32) {
     extern __shared__ float lds[];
     float *qf = lds;                        // [H * d]
     float *tk = qf + H * d;                 // [H * H]
     float *s = tk + H * H;                  // [H][64] capped scores
     float *p = s + H * kWaChunk;            // [H][64] softmax numerators
     float *alpha = p + H * kWaChunk;        // [H]
-    float *lsum = alpha + H;                // [H]
     int64_t *kbase = reinterpret_cast<int64_t *>(lds + wa_float_count(H, d));   // [64] block id of each key (8-byte aligned)
     int *koff = reinterpret_cast<int *>(kbase + kWaChunk);                          // [64] slot inside the block
 
@@ -47,7 +54,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int pos = tok_pos[t];
     const int32_t *bt = block_table + static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq;
-    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int lo = window <= 0 ? 0 : mask_kind == 1 ? (pos / window) * window : (pos - window + 1 > 0 ? pos - window + 1 : 0);
     const int nkeys = pos - lo + 1;
     const int rep = H / G;
 
@@ -117,10 +124,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
             lrun[i] = lrun[i] * al + csum;
             mrun[i] = mnew;
             p[h * kWaChunk + lane] = pj;
-            if (lane == 0) {
-                alpha[h] = al;
-                lsum[h] = lrun[i];
-            }
+            if (lane == 0) alpha[h] = al;
         }
         __syncthreads();
         // 3. weighted values
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
             const int idx = tid + i * kWaThreads;
             if (idx < H * dv) {
                 const int h = idx / dv, col = idx - h * dv;
-                const int g = h / rep;
+                const int g = (h / rep) % GV;
                 float a = acc[i] * alpha[h];
                 const float *ph = p + h * kWaChunk;
                 for (int j = 0; j < cn; ++j) {
@@ -143,12 +147,30 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
         }
     }
     __syncthreads();
-    T *orow = out + t * static_cast<int64_t>(H) * dv;
+    // final scale of every head: 1 / sum, or with a sink e^(m - M) / (sum e^(m - M) + e^(sink - M)), M = max(m, sink)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int h = wave + 4 * i;
+        if (i >= hpw || h >= H) break;
+        float al = 1.f, l = lrun[i];
+        if (sink) {
+            const float sk = sink[h], big = fmaxf(mrun[i], sk);
+            al = expf(mrun[i] - big);
+            l = l * al + expf(sk - big);
+        }
+        if (lane == 0) alpha[h] = al / l;
+    }
+    __syncthreads();
+    const int64_t obase = t * static_cast<int64_t>(H) * dv;
 #pragma unroll
     for (int i = 0; i < kWaMaxAcc; ++i) {
         if (i >= nacc) break;
         const int idx = tid + i * kWaThreads;
-        if (idx < H * dv) orow[idx] = to_t<T>(acc[i] / lsum[idx / dv]);
+        if (idx < H * dv) {
+            const float o = acc[i] * alpha[idx / dv];
+            if (out_f32) reinterpret_cast<float *>(out)[obase + idx] = o;
+            else out[obase + idx] = to_t<T>(o);
+        }
     }
 }
 
@@ -158,16 +180,18 @@ inline size_t wa_lds_bytes(int H, int d) {
 
 } // namespace swl
 
-extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache,
+extern "C" int swl_masked_attn(void *out, const void *q, const void *k_cache, const void *v_cache,
                                const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
                                const float *talk, const float *rel, int32_t rel_len, int64_t num_tokens,
                                int32_t num_q_heads, int32_t num_kv_heads,
                                int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window, float scale,
-                               float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                               float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t mask_kind,
+                               const float *sink, int32_t num_v_heads, int32_t out_f32, int32_t dtype,
                                swl_stream_t stream) {
     if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || dim <= 0 || vdim <= 0 || window < 0)
         return SWL_ERR_BAD_ARG;
     if (num_q_heads % num_kv_heads) return SWL_ERR_BAD_ARG;
+    if (mask_kind < 0 || mask_kind > 1 || num_v_heads <= 0 || num_kv_heads % num_v_heads) return SWL_ERR_BAD_ARG;
     if (num_tokens == 0) return SWL_OK;
     if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || (rel && rel_len <= 0))
         return SWL_ERR_BAD_ARG;
@@ -181,7 +205,19 @@ extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, co
                            static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, tok_seq,
                            tok_pos, talk, rel, rel_len, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale,
                            softcap,
-                           max_blocks_per_seq, block_stride);
+                           max_blocks_per_seq, block_stride, mask_kind, sink, num_v_heads, out_f32);
     });
     return swl::check_launch();
+}
+
+extern "C" int swl_window_attn(void *out, const void *q, const void *k_cache, const void *v_cache,
+                               const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                               const float *talk, const float *rel, int32_t rel_len, int64_t num_tokens,
+                               int32_t num_q_heads, int32_t num_kv_heads,
+                               int32_t dim, int32_t vdim, int64_t q_tok_stride, int32_t window, float scale,
+                               float softcap, int32_t max_blocks_per_seq, int64_t block_stride, int32_t dtype,
+                               swl_stream_t stream) {
+    return swl_masked_attn(out, q, k_cache, v_cache, block_table, tok_seq, tok_pos, talk, rel, rel_len, num_tokens,
+                           num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale, softcap, max_blocks_per_seq,
+                           block_stride, 0, nullptr, num_kv_heads > 0 ? num_kv_heads : 1, 0, dtype, stream);
 }

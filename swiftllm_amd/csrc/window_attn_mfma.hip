@@ -11,6 +11,11 @@
 //      every weight although the matrix core takes 16-bit operands.
 // The transposed products keep the query index on the lanes' low four bits in every stage, so the softmax statistics of a
 // query never move between lanes. Keys outside [pos - window + 1, pos] get weight zero; pages wholly outside are skipped.
+//
+// The general entry point (swl_masked_attn_tiles) adds: mask_kind 1 (chunked visibility: keys [floor(p / window) * window, p]),
+// sink[H] (a logit per head that joins the denominator only), num_v_heads (value head = key head % num_v_heads: score maps
+// that share their values), out_f32 (fp32 result), and a split of the heads over blockIdx.z (head_groups: every group of
+// heads_per_group heads is a workgroup of its own — many heads over one shared key head, wide value heads).
 #include "swl_common.h"
 
 namespace swl {
@@ -25,7 +30,8 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk,
     const float *__restrict__ rel, int rel_len, int H, int G,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
-    float *part_o, float *part_ml, int64_t num_tokens, int nbuf) {
+    float *part_o, float *part_ml, int64_t num_tokens, int nbuf, int mask_kind, const float *__restrict__ sink, int GV,
+    int out_f32, int hpg) {
     // [nbuf][H][64 lanes][4] capped scores of a page, then [H][H] the mixing matrix. nbuf = 2: pages alternate between two
     // score buffers and ONE barrier per page suffices (a wave that is a page ahead writes the other buffer)
     extern __shared__ float s_all[];
@@ -47,10 +53,14 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     const int p0 = __builtin_amdgcn_readfirstlane(tok_pos[row0]);
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
     const int rep = H / G;
-    const int h0 = wave * HPW;
+    // heads of this workgroup: [hbase, hend); wave w owns HPW of them
+    const int hbase = static_cast<int>(blockIdx.z) * hpg, hend = min(H, hbase + hpg);
+    const int h0 = hbase + wave * HPW;
     const int qpos = p0 + li;                        // this lane's query position (meaningful when li < cnt)
     const bool qok = li < cnt;
-    const int lo_first = (window > 0 && p0 - window + 1 > 0) ? p0 - window + 1 : 0;
+    // first visible key of this lane's query, and of the tile's first query
+    const int qlo = window <= 0 ? 0 : mask_kind == 1 ? (qpos / window) * window : qpos - window + 1;
+    const int lo_first = window <= 0 ? 0 : mask_kind == 1 ? (p0 / window) * window : (p0 - window + 1 > 0 ? p0 - window + 1 : 0);
     int kb0 = lo_first / kWmTile, kb1 = (p0 + cnt - 1) / kWmTile;
     if (gridDim.y > 1) {    // key split: this workgroup takes a contiguous share of the tile's pages (possibly none)
         const int per = (kb1 - kb0 + static_cast<int>(gridDim.y)) / static_cast<int>(gridDim.y);
@@ -82,7 +92,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     for (int hh = 0; hh < HPW; ++hh) {
         const int kv = __builtin_amdgcn_readfirstlane(min(h0 + hh, H - 1) / rep);
         koff[hh] = kv * kWmTile * D;
-        voff[hh] = kv * DV * kWmTile;
+        voff[hh] = (kv % GV) * DV * kWmTile;
     }
     const int lane_k = li * D + 4 * lq;             // A operand of S^T: key li, dims 4 lq ..
     const int lane_v = li * kWmTile + 4 * lq;       // A operand of O^T: column li of a 16-column tile, keys 4 lq ..
@@ -133,7 +143,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int g = h0 + hh;
-            if (g < H) {
+            if (g < hend) {
                 float4_t st = {0.f, 0.f, 0.f, 0.f};
                 if constexpr (PIPE) {
 #pragma unroll
@@ -177,7 +187,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int kp = kpos0 + r;
-            ok[r] = qok && kp <= qpos && (window <= 0 || kp > qpos - window);
+            ok[r] = qok && kp <= qpos && kp >= qlo;
         }
         for (int g = 0; MIX && g < H; ++g) {
             const float4_t sv = *reinterpret_cast<const float4_t *>(&s_lds[(g * 64 + lane) * 4]);
@@ -201,7 +211,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
 #pragma unroll
         for (int hh = 0; hh < HPW; ++hh) {
             const int h = h0 + hh;
-            if (h < H) {
+            if (h < hend) {
                 float cmax = kNegBig;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) cmax = fmaxf(cmax, ok[r] ? mixed[hh][r] : kNegBig);
@@ -246,7 +256,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
 #pragma unroll
     for (int hh = 0; hh < HPW; ++hh) {
         const int h = h0 + hh;
-        if (h < H) {
+        if (h < hend) {
             float l = lrun[hh];
             l += __shfl_xor(l, 16, 64);
             l += __shfl_xor(l, 32, 64);
@@ -264,17 +274,29 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
                 }
                 continue;
             }
-            const float inv = 1.0f / l;
+            float inv = 1.0f / l;
+            if (sink) {     // the sink joins the denominator: rebase the row on max(m, sink) (base-2 units)
+                const float sk = sink[h] * kLog2e, big = fmaxf(mrun[hh], sk);
+                const float a = fast_exp2(mrun[hh] - big);
+                inv = a / (l * a + fast_exp2(sk - big));
+            }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 float4_t o = acc[hh][ct];
                 mfma_results_ready<4>(o);
                 if (qok) {
-                    typedef T vec4 __attribute__((ext_vector_type(4)));
-                    vec4 w;
+                    const int64_t at = (static_cast<int64_t>(row0 + li) * H + h) * DV + ct * 16 + 4 * lq;
+                    if (out_f32) {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) w[r] = to_t<T>(o[r] * inv);
-                    *reinterpret_cast<vec4 *>(out + (static_cast<int64_t>(row0 + li) * H + h) * DV + ct * 16 + 4 * lq) = w;
+                        for (int r = 0; r < 4; ++r) o[r] *= inv;
+                        *reinterpret_cast<float4_t *>(reinterpret_cast<float *>(out) + at) = o;
+                    } else {
+                        typedef T vec4 __attribute__((ext_vector_type(4)));
+                        vec4 w;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) w[r] = to_t<T>(o[r] * inv);
+                        *reinterpret_cast<vec4 *>(out + at) = w;
+                    }
                 }
             }
         }
@@ -284,33 +306,43 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
 // out[t][h][:] = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s over the key shares s (a share without keys has l = 0)
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_combine_kernel(T *out, const float *part_o, const float *part_ml,
-                                                                  int64_t rows, int dv, int nsplit) {
+                                                                  int64_t rows, int dv, int nsplit, const float *sink, int H,
+                                                                  int out_f32) {
     const int64_t row = blockIdx.x;     // (token, head)
     float mx = kNegBig;     // (the maxima are in base-2 exponent units)
     for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(s * rows + row) * 2]);
     float den = 0.f;
+    if (sink) {
+        const float sk = sink[row % H] * 1.4426950408889634f;
+        mx = fmaxf(mx, sk);
+        den = exp2f(sk - mx);
+    }
     for (int s = 0; s < nsplit; ++s)
         den += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_ml[(s * rows + row) * 2 + 1];
     for (int c = threadIdx.x; c < dv; c += blockDim.x) {
         float a = 0.f;
         for (int s = 0; s < nsplit; ++s)
             a += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_o[(s * rows + row) * dv + c];
-        out[row * dv + c] = to_t<T>(a / den);
+        if (out_f32) reinterpret_cast<float *>(out)[row * dv + c] = a / den;
+        else out[row * dv + c] = to_t<T>(a / den);
     }
 }
 
-template <typename T, int D, int DV>
+template <typename T, int D, int DV, bool MIXOK>
 int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q, const T *kc, const T *vc,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
               const float *talk, const float *rel, int rel_len, int H, int G, int64_t qs, int window, float scale,
               float softcap, int mb, int64_t bs,
-              float *po, float *pml, int64_t nt, int nbuf) {
+              float *po, float *pml, int64_t nt, int nbuf, int mask_kind, const float *sink, int GV, int out_f32, int hpg) {
 #define SWL_WM_LAUNCH1(HPW, NW, MIX)                                                                                         \
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW, MIX>), grid, dim3(NW * 64), MIX ? lds : 0, s, out, q, kc, \
-                       vc, bt, ts, tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf)
-#define SWL_WM_LAUNCH(HPW, NW)          \
-    if (talk) SWL_WM_LAUNCH1(HPW, NW, true); \
-    else SWL_WM_LAUNCH1(HPW, NW, false)
+                       vc, bt, ts, tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf, mask_kind,  \
+                       sink, GV, out_f32, hpg)
+#define SWL_WM_LAUNCH(HPW, NW)                                 \
+    if (talk) {                                                \
+        if constexpr (MIXOK) SWL_WM_LAUNCH1(HPW, NW, true);    \
+        else return SWL_ERR_UNSUPPORTED;                       \
+    } else SWL_WM_LAUNCH1(HPW, NW, false)
     // heads per wave x waves: up to 16 heads on four waves, more on eight (four heads per wave at most: the accumulators of
     // eight 128-wide heads do not fit a wave's registers)
     switch (hpw) {
@@ -325,20 +357,102 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
     if (grid.y > 1) {
         const int64_t rows = nt * H;
         hipLaunchKernelGGL((window_attn_combine_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(DV < 256 ? 64 : 256), 0, s,
-                           out, po, pml, rows, DV, static_cast<int>(grid.y));
+                           out, po, pml, rows, DV, static_cast<int>(grid.y), sink, H, out_f32);
     }
     return check_launch();
 }
 
 } // namespace swl
 
+// (dim, vdim) pairs with a compiled kernel; the first four also with the head-mixing matrix
+#define SWL_WM_SHAPES_MIX(X) X(64, 64) X(128, 128) X(128, 64) X(64, 128)
+#define SWL_WM_SHAPES_PLAIN(X) \
+    X(32, 32) X(32, 64) X(48, 48) X(48, 96) X(64, 32) X(64, 96) X(96, 64) X(96, 96) X(128, 96) X(96, 128) X(160, 128) X(192, 128)
+
+static int wm_shape_kind(int dim, int vdim) {      // 2: with or without mixing, 1: without only, 0: none
+#define SWL_WM_IS(DD, DDV) if (dim == DD && vdim == DDV) return 2;
+    SWL_WM_SHAPES_MIX(SWL_WM_IS)
+#undef SWL_WM_IS
+#define SWL_WM_IS(DD, DDV) if (dim == DD && vdim == DDV) return 1;
+    SWL_WM_SHAPES_PLAIN(SWL_WM_IS)
+#undef SWL_WM_IS
+    return 0;
+}
+
 /* 1 when swl_window_attn_tiles serves this shape (else the caller uses swl_window_attn). */
 extern "C" int swl_window_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim,
                                                int32_t dtype) {
     if (dtype != SWL_F16 && dtype != SWL_BF16) return 0;
     if (num_q_heads <= 0 || num_q_heads > 32 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
-    return (dim == 64 && vdim == 64) || (dim == 128 && vdim == 128) || (dim == 128 && vdim == 64) ||
-           (dim == 64 && vdim == 128);
+    return wm_shape_kind(dim, vdim) == 2;
+}
+
+/* 1 when swl_masked_attn_tiles serves this shape without a head-mixing matrix. More than 32 heads are served when the
+ * heads can be split into groups (no mixing), 32 at most per workgroup. */
+extern "C" int swl_masked_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t num_v_heads, int32_t dim,
+                                               int32_t vdim, int32_t dtype) {
+    if (dtype != SWL_F16 && dtype != SWL_BF16) return 0;
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads) return 0;
+    if (num_v_heads <= 0 || num_kv_heads % num_v_heads) return 0;
+    return wm_shape_kind(dim, vdim) > 0;
+}
+
+extern "C" int swl_masked_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                     const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                                     const int32_t *tile_row0, const int32_t *tile_cnt, const float *talk,
+                                     const float *rel, int32_t rel_len, int32_t num_tiles, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                                     int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, float softcap,
+                                     int32_t max_blocks_per_seq, int64_t block_stride, int32_t key_splits,
+                                     float *scratch, int64_t num_tokens, int32_t mask_kind, const float *sink,
+                                     int32_t num_v_heads, int32_t out_f32, int32_t heads_per_group, int32_t dtype,
+                                     swl_stream_t stream) {
+    if (num_tiles < 0 || window < 0 || key_splits < 1 || key_splits > 64) return SWL_ERR_BAD_ARG;
+    if (key_splits > 1 && (!scratch || num_tokens <= 0 || (reinterpret_cast<uintptr_t>(scratch) & 15)))
+        return SWL_ERR_BAD_ARG;
+    if (mask_kind < 0 || mask_kind > 1 || heads_per_group < 0) return SWL_ERR_BAD_ARG;
+    if (!swl_masked_attn_tiles_supported(num_q_heads, num_kv_heads, num_v_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
+    // heads per workgroup: all of them when they are mixed (the mix couples them), else the caller's choice (0: all)
+    int hpg = (talk || heads_per_group == 0) ? num_q_heads : (heads_per_group < num_q_heads ? heads_per_group : num_q_heads);
+    if (hpg > 32) {
+        if (talk) return SWL_ERR_UNSUPPORTED;
+        hpg = 32;
+    }
+    if (num_tiles == 0) return SWL_OK;
+    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt ||
+        (rel && rel_len <= 0))
+        return SWL_ERR_BAD_ARG;
+    if ((q_tok_stride & 3) || (block_stride & 3) || (reinterpret_cast<uintptr_t>(q) & 7) ||
+        (reinterpret_cast<uintptr_t>(k_cache) & 7) || (reinterpret_cast<uintptr_t>(v_cache) & 7) ||
+        (reinterpret_cast<uintptr_t>(out) & (out_f32 ? 15 : 7)))
+        return SWL_ERR_BAD_ARG;     // 8-byte operand loads
+    int hpw = (hpg + swl::kWmWaves - 1) / swl::kWmWaves;
+    hpw = hpw <= 1 ? 1 : hpw <= 2 ? 2 : hpw <= 4 ? 4 : 8;
+    const int groups = (num_q_heads + hpg - 1) / hpg;
+    const size_t one = static_cast<size_t>(num_q_heads) * 256, mixw = static_cast<size_t>(num_q_heads) * num_q_heads;
+    const int nbuf = (2 * one + mixw) * sizeof(float) <= 64 * 1024 ? 2 : 1;
+    const size_t lds = (nbuf * one + mixw) * sizeof(float);
+    const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(key_splits), static_cast<unsigned>(groups));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // scratch: [splits][tokens][H][vdim] fp32 partial outputs, then [splits][tokens][H][2] (maximum, sum)
+    float *part_o = scratch;
+    float *part_ml = scratch ? scratch + static_cast<int64_t>(key_splits) * num_tokens * num_q_heads * vdim : nullptr;
+#define SWL_WM_SHAPE_(DD, DDV, MIXOK)                                                                                     \
+    if (dim == DD && vdim == DDV)                                                                                         \
+        return swl::launch_wm<T, DD, DDV, MIXOK>(hpw, grid, lds, s, static_cast<T *>(out), static_cast<const T *>(q),    \
+                                          static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
+                                          tok_seq, tok_pos, tile_row0, tile_cnt, talk, rel, rel_len, num_q_heads, num_kv_heads, \
+                                          q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
+                                          part_ml, num_tokens, nbuf, mask_kind, sink, num_v_heads, out_f32, hpg);
+#define SWL_WM_SHAPE_MIX(DD, DDV) SWL_WM_SHAPE_(DD, DDV, true)
+#define SWL_WM_SHAPE_PLAIN(DD, DDV) SWL_WM_SHAPE_(DD, DDV, false)
+    SWL_DISPATCH_DTYPE(dtype, T, {
+        SWL_WM_SHAPES_MIX(SWL_WM_SHAPE_MIX)
+        SWL_WM_SHAPES_PLAIN(SWL_WM_SHAPE_PLAIN)
+    });
+#undef SWL_WM_SHAPE_
+#undef SWL_WM_SHAPE_MIX
+#undef SWL_WM_SHAPE_PLAIN
+    return SWL_ERR_UNSUPPORTED;
 }
 
 extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache,
@@ -348,40 +462,9 @@ extern "C" int swl_window_attn_tiles(void *out, const void *q, const void *k_cac
                                      int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, float softcap,
                                      int32_t max_blocks_per_seq, int64_t block_stride, int32_t key_splits,
                                      float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream) {
-    if (num_tiles < 0 || window < 0 || key_splits < 1 || key_splits > 64) return SWL_ERR_BAD_ARG;
-    if (key_splits > 1 && (!scratch || num_tokens <= 0 || (reinterpret_cast<uintptr_t>(scratch) & 15)))
-        return SWL_ERR_BAD_ARG;
     if (!swl_window_attn_tiles_supported(num_q_heads, num_kv_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
-    if (num_tiles == 0) return SWL_OK;
-    if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt ||
-        (rel && rel_len <= 0))
-        return SWL_ERR_BAD_ARG;
-    if ((q_tok_stride & 3) || (block_stride & 3) || (reinterpret_cast<uintptr_t>(q) & 7) ||
-        (reinterpret_cast<uintptr_t>(k_cache) & 7) || (reinterpret_cast<uintptr_t>(out) & 7))
-        return SWL_ERR_BAD_ARG;     // 8-byte operand loads
-    int hpw = (num_q_heads + swl::kWmWaves - 1) / swl::kWmWaves;
-    hpw = hpw <= 1 ? 1 : hpw <= 2 ? 2 : hpw <= 4 ? 4 : 8;
-    const size_t one = static_cast<size_t>(num_q_heads) * 256, mixw = static_cast<size_t>(num_q_heads) * num_q_heads;
-    const int nbuf = (2 * one + mixw) * sizeof(float) <= 64 * 1024 ? 2 : 1;
-    const size_t lds = (nbuf * one + mixw) * sizeof(float);
-    const dim3 grid(static_cast<unsigned>(num_tiles), static_cast<unsigned>(key_splits));
-    hipStream_t s = static_cast<hipStream_t>(stream);
-    // scratch: [splits][tokens][H][vdim] fp32 partial outputs, then [splits][tokens][H][2] (maximum, sum)
-    float *part_o = scratch;
-    float *part_ml = scratch ? scratch + static_cast<int64_t>(key_splits) * num_tokens * num_q_heads * vdim : nullptr;
-#define SWL_WM_SHAPE(DD, DDV)                                                                                             \
-    if (dim == DD && vdim == DDV)                                                                                         \
-        return swl::launch_wm<T, DD, DDV>(hpw, grid, lds, s, static_cast<T *>(out), static_cast<const T *>(q),           \
-                                          static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
-                                          tok_seq, tok_pos, tile_row0, tile_cnt, talk, rel, rel_len, num_q_heads, num_kv_heads, \
-                                          q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
-                                          part_ml, num_tokens, nbuf);
-    SWL_DISPATCH_DTYPE(dtype, T, {
-        SWL_WM_SHAPE(64, 64)
-        SWL_WM_SHAPE(128, 128)
-        SWL_WM_SHAPE(128, 64)
-        SWL_WM_SHAPE(64, 128)
-    });
-#undef SWL_WM_SHAPE
-    return SWL_ERR_UNSUPPORTED;
+    return swl_masked_attn_tiles(out, q, k_cache, v_cache, block_table, tok_seq, tok_pos, tile_row0, tile_cnt, talk, rel,
+                                 rel_len, num_tiles, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale,
+                                 softcap, max_blocks_per_seq, block_stride, key_splits, scratch, num_tokens, 0, nullptr,
+                                 num_kv_heads, 0, 0, dtype, stream);
 }

@@ -327,3 +327,168 @@ class LorulixModelConfig:
     def load_from_model_path(model_path: str) -> "LorulixModelConfig":
         with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
             return LorulixModelConfig(json.load(f))
+
+
+# ---- Rosilix ---------------------------------------------------------------------------------------------------------------
+class RotaryConfig:
+    """Rotary positions on interleaved pairs: dimension 2i of a head turns with dimension 2i + 1 by the angle
+    position * base^(-2i / dims), for i < dims / 2; the dimensions from `dims` on pass unchanged."""
+
+    def __init__(self, rot: dict, head_dim: int):
+        self.dims = int(rot["dims"]) if rot else 0
+        self.base = float(rot["base"]) if rot else 1.0
+        if self.dims < 0 or self.dims % 2 or self.dims > head_dim:
+            raise ValueError(f"rot.dims ({self.dims}) must be even and at most the head size ({head_dim})")
+
+    def frequencies(self):
+        """base^(-2i / dims) for i < dims / 2, in float64."""
+        return [self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)]
+
+
+class RosilixDiffAttentionConfig:
+    """Differential attention: every head holds two score maps (queries and keys of 2 * dim, laid out [map 1 | map 2]) over
+    the same values; the maps' outputs are combined as a1 - lambda * a2, brought to unit RMS per head, scaled by 1 - diff
+    and gated per head. Keys are visible inside the query's own chunk of `chunk` positions (0: every earlier key)."""
+    kind = "attention"
+
+    def __init__(self, mixer: dict):
+        self.num_q_heads = int(mixer["heads"])
+        self.num_kv_heads = int(mixer.get("kv_heads", self.num_q_heads))
+        self.head_dim = int(mixer["dim"])                       # of one map
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.scale = float(mixer["scale"])
+        self.diff = float(mixer["diff"])
+        mask = mixer.get("mask") or {}
+        self.chunk = int(mask["size"]) if mask.get("size") else 0
+        self.rot = RotaryConfig(mixer.get("rot"), self.head_dim)
+        self.kv_from = -1
+        if self.num_q_heads % self.num_kv_heads:
+            raise ValueError(f"heads ({self.num_q_heads}) must be a multiple of kv_heads ({self.num_kv_heads})")
+        if self.head_dim % 2:
+            raise ValueError(f"dim ({self.head_dim}) must be even")
+
+    @property
+    def q_size(self) -> int:
+        return 2 * self.num_q_heads * self.head_dim
+
+    @property
+    def k_size(self) -> int:
+        return 2 * self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def o_size(self) -> int:
+        return self.num_q_heads * self.value_dim
+
+
+class RosilixLatentAttentionConfig:
+    """Latent attention: keys and values of all heads are up-projections of one cached latent row of `kv_rank` per token,
+    plus one rotated key part of `rot_dim` shared by the heads; a learned sink per head joins the softmax denominator; the
+    heads are gated. `kv_from` >= 0: the layer has no compression of its own and reads that layer's cached rows."""
+    kind = "latent_attention"
+
+    def __init__(self, mixer: dict):
+        self.num_q_heads = int(mixer["heads"])
+        self.num_kv_heads = 1
+        self.head_dim = int(mixer["dim"])                       # unrotated part of a query / key head
+        self.rot_dim = int(mixer["rot_dim"])
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.kv_rank = int(mixer["kv_rank"])
+        self.scale = float(mixer["scale"])
+        self.rot = RotaryConfig(mixer["rot"], self.rot_dim)
+        self.kv_from = int(mixer["kv_from"]) if mixer.get("kv_from") is not None else -1
+        if self.rot.dims != self.rot_dim:
+            raise ValueError(f"rot.dims ({self.rot.dims}) must equal rot_dim ({self.rot_dim})")
+
+    @property
+    def q_size(self) -> int:
+        return self.num_q_heads * (self.head_dim + self.rot_dim)
+
+    @property
+    def dkv_size(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def k_size(self) -> int:
+        """Elements of the cached key row: the latent and the shared rotated part."""
+        return self.kv_rank + self.rot_dim
+
+    @property
+    def v_size(self) -> int:
+        """Elements of the cached value row: the latent once more (kept transposed for the value product)."""
+        return self.kv_rank
+
+    @property
+    def o_size(self) -> int:
+        return self.num_q_heads * self.value_dim
+
+
+class RosilixMlpConfig:
+    """`dense`: down(relu(up h)^2)."""
+
+    def __init__(self, mlp: dict):
+        self.kind = mlp["kind"]
+        if self.kind != "dense":
+            raise ValueError(f"unsupported mlp.kind {self.kind!r}")
+        self.ffn_inter_dim = int(mlp["ff"])
+
+
+class RosilixLayerConfig:
+    def __init__(self, layer: dict):
+        self.type = layer["type"]
+        if self.type == "attention":
+            self.mixer = RosilixDiffAttentionConfig(layer["mixer"])
+        elif self.type == "latent_attention":
+            self.mixer = RosilixLatentAttentionConfig(layer["mixer"])
+        else:
+            raise ValueError(f"unsupported layer type {self.type!r}")
+        self.mlp = RosilixMlpConfig(layer["mlp"]) if layer.get("mlp") else None
+
+
+class RosilixModelConfig:
+    """Rosilix: a decoder-only model with an fp32 stream, RMS norms before and after every sublayer, rotary positions on
+    interleaved pairs, and two kinds of mixer in any order: chunked differential attention and latent attention with a
+    softmax sink (a layer may read an earlier latent layer's cache). Feed-forwards are squared-ReLU. Every size and constant
+    is read from config.json. The design has no position table: `max_positions`, if config.json gives it, bounds a sequence;
+    otherwise the bound is DEFAULT_MAX_POSITIONS."""
+    DEFAULT_MAX_POSITIONS = 1 << 20
+
+    def __init__(self, model_config: dict):
+        if model_config.get("architecture") != "Rosilix":
+            raise AssertionError(f"unsupported architecture {model_config.get('architecture')!r}")
+        self.vocab_size = int(model_config["vocab"])
+        self.hidden_size = int(model_config["width"])
+        self.max_position_embeddings = int(model_config.get("max_positions") or self.DEFAULT_MAX_POSITIONS)
+        self.norm_eps = float(model_config["norm"]["eps"])
+        self.embedding_scale = float((model_config.get("embedding") or {}).get("scale", 1.0))
+        self.layers = [RosilixLayerConfig(layer) for layer in model_config["layers"]]
+        self.num_layers = len(self.layers)
+        for i, layer in enumerate(self.layers):
+            j = layer.mixer.kv_from
+            if j < 0:
+                continue
+            src = self.layers[j] if 0 <= j < i else None
+            if src is None or src.type != "latent_attention" or src.mixer.kv_from >= 0:
+                raise ValueError(f"layer {i}: kv_from {j} must name an earlier latent attention layer with a cache of its own")
+            a, b = layer.mixer, src.mixer
+            if (a.kv_rank, a.rot_dim, a.rot.base) != (b.kv_rank, b.rot_dim, b.rot.base):
+                raise ValueError(f"layer {i}: latent size or rotation differ from those of layer {j}")
+        # what the scheduler-facing code reads off any model's configuration
+        self.num_q_heads = max(l.mixer.num_q_heads for l in self.layers)
+        self.num_kv_heads = max(l.mixer.num_kv_heads for l in self.layers)
+        self.head_dim = max(l.mixer.head_dim for l in self.layers)
+
+    def kv_elems_per_token(self) -> int:
+        """Cached elements per token over the layers that keep a cache of their own."""
+        return sum(l.mixer.k_size + l.mixer.v_size for l in self.layers if l.mixer.kv_from < 0)
+
+    def get_kvslot_size(self, dtype: torch.dtype = torch.bfloat16) -> int:
+        return max(self.kv_elems_per_token(), 1) * dtype.itemsize
+
+    @staticmethod
+    def load_from_model_path(model_path: str) -> "RosilixModelConfig":
+        with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
+            return RosilixModelConfig(json.load(f))

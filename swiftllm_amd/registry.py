@@ -13,6 +13,7 @@ MODELS = {
     "llama": ("swiftllm_amd.model_config:LlamaModelConfig", "swiftllm_amd.worker.model:LlamaModel"),
     "Kekapel": ("swiftllm_amd.model_config:KekapelModelConfig", "swiftllm_amd.worker.kekapel_model:KekapelModel"),
     "Lorulix": ("swiftllm_amd.model_config:LorulixModelConfig", "swiftllm_amd.worker.lorulix_model:LorulixModel"),
+    "Rosilix": ("swiftllm_amd.model_config:RosilixModelConfig", "swiftllm_amd.worker.rosilix_model:RosilixModel"),
 }
 
 

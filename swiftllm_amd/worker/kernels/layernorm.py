@@ -7,11 +7,14 @@ from swiftllm_amd import _hip
 
 def embed_positions(tokens: torch.Tensor, positions: torch.Tensor, embed: torch.Tensor, pos: torch.Tensor, scale: float,
                     keep_copy: bool):
-    """-> (x fp32 [T, width], copy of it or None): x[t] = embed[tokens[t]] * scale + pos[positions[t]]."""
+    """-> (x fp32 [T, width], copy of it or None): x[t] = embed[tokens[t]] * scale + pos[positions[t]] (pos None: a model
+    without learned positions)."""
     _hip.require_gpu_tensor(embed, "embed")
     n, width = tokens.shape[0], embed.shape[1]
-    assert embed.is_contiguous() and pos.is_contiguous() and pos.shape[1] == width and embed.dtype == pos.dtype
-    assert tokens.dtype == torch.int32 and positions.dtype == torch.int32 and positions.shape[0] == n
+    assert embed.is_contiguous() and tokens.dtype == torch.int32
+    if pos is not None:
+        assert pos.is_contiguous() and pos.shape[1] == width and embed.dtype == pos.dtype
+        assert positions.dtype == torch.int32 and positions.shape[0] == n
     x = torch.empty((n, width), dtype=torch.float32, device=embed.device)
     x0 = torch.empty_like(x) if keep_copy else None
     _hip.call("swl_embed_pos", _hip.ptr(x), _hip.ptr(x0), _hip.ptr(embed), _hip.ptr(pos), _hip.ptr(tokens),

@@ -135,3 +135,78 @@ def window_attention(qkv: torch.Tensor, talk: torch.Tensor, pool: torch.Tensor, 
               mixer.window, float(mixer.scale), float(mixer.softcap), block_table.shape[1], pool.shape[1],
               _hip.dtype_code3(qkv.dtype), _hip.stream())
     return out
+
+
+# ---- the same loops with other masks and denominators -----------------------------------------------------------------------
+MASK_WINDOW = 0     # keys [p - window + 1, p]
+MASK_CHUNK = 1      # keys [floor(p / window) * window, p]
+
+
+class AttentionSpec:
+    """Shape and constants of one attention over the pool, as the kernels see it (which need not be how the design counts
+    its heads: two score maps over shared values are 2 H query heads, 2 G key heads and G value heads).
+    num_v_heads: value heads in a page; key head g reads value head g % num_v_heads. window: sliding window or chunk size
+    (mask_kind), 0 for every earlier key. sink: fp32 [num_q_heads] logits that join the denominators, or None."""
+    __slots__ = ("num_q_heads", "num_kv_heads", "num_v_heads", "head_dim", "value_dim", "window", "mask_kind", "scale",
+                 "softcap", "sink", "out_f32")
+
+    def __init__(self, num_q_heads, num_kv_heads, head_dim, value_dim, scale, window=0, mask_kind=MASK_WINDOW,
+                 num_v_heads=None, softcap=0.0, sink=None, out_f32=False):
+        self.num_q_heads, self.num_kv_heads, self.head_dim, self.value_dim = num_q_heads, num_kv_heads, head_dim, value_dim
+        self.num_v_heads = num_kv_heads if num_v_heads is None else num_v_heads
+        self.window, self.mask_kind, self.scale, self.softcap, self.sink, self.out_f32 = \
+            window, mask_kind, scale, softcap, sink, out_f32
+
+
+def masked_tiles_supported(spec: AttentionSpec, dtype: torch.dtype) -> bool:
+    if dtype not in (torch.float16, torch.bfloat16):
+        return False
+    return bool(_hip.load().swl_masked_attn_tiles_supported(spec.num_q_heads, spec.num_kv_heads, spec.num_v_heads,
+                                                            spec.head_dim, spec.value_dim, _hip.dtype_code(dtype)))
+
+
+def choose_heads_per_group(spec: AttentionSpec) -> int:
+    """Heads of one workgroup of the matrix-core kernel (four waves): as many per wave as keep a wave's query, key and value
+    fragments and accumulators in registers, so that many or wide heads are shared out over several workgroups."""
+    per_wave = max(1, 512 // (spec.head_dim + spec.value_dim))
+    per_wave = 4 if per_wave >= 4 else 2 if per_wave >= 2 else 1
+    return min(spec.num_q_heads, 4 * per_wave)
+
+
+def masked_attention(q: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice, block_table: torch.Tensor,
+                     tok_seq: torch.Tensor, tok_pos: torch.Tensor, spec: AttentionSpec, tiles=None,
+                     max_positions: int = 1 << 20) -> torch.Tensor:
+    """-> [T, num_q_heads * value_dim] (fp32 when spec.out_f32, else q's dtype). q: rows whose first num_q_heads * head_dim
+    columns are the queries (a column slice of a wider matrix is fine); keys and values come from the pool, which already
+    holds this step's tokens."""
+    _hip.require_gpu_tensor(q, "q")
+    assert q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= spec.num_q_heads * spec.head_dim
+    assert pool.is_contiguous() and pool.dtype == q.dtype and tok_pos.dtype == torch.int32 and tok_seq.dtype == torch.int32
+    sink = spec.sink
+    assert sink is None or (sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == spec.num_q_heads)
+    n = q.shape[0]
+    out = torch.empty((n, spec.num_q_heads * spec.value_dim), dtype=torch.float32 if spec.out_f32 else q.dtype,
+                      device=q.device)
+    esize = pool.element_size()
+    kp = pool.data_ptr() + pool_slice.k_offset * esize
+    vp = pool.data_ptr() + pool_slice.v_offset * esize
+    wide_ok = q.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0 and kp % 8 == 0 and vp % 8 == 0 and pool.shape[1] % 4 == 0
+    if tiles is not None and wide_ok and masked_tiles_supported(spec, q.dtype):
+        row0, cnt = tiles
+        hpg = choose_heads_per_group(spec)
+        groups = -(-spec.num_q_heads // hpg)
+        splits = choose_key_splits(row0.shape[0] * groups, spec, max_positions)
+        scratch = None
+        if splits > 1:
+            scratch = _split_scratch(q.device, splits * n * spec.num_q_heads * (spec.value_dim + 2))
+        _hip.call("swl_masked_attn_tiles", _hip.ptr(out), _hip.ptr(q), kp, vp, _hip.ptr(block_table), _hip.ptr(tok_seq),
+                  _hip.ptr(tok_pos), _hip.ptr(row0), _hip.ptr(cnt), 0, 0, 0, row0.shape[0], spec.num_q_heads,
+                  spec.num_kv_heads, spec.head_dim, spec.value_dim, q.stride(0), spec.window, float(spec.scale),
+                  float(spec.softcap), block_table.shape[1], pool.shape[1], splits, _hip.ptr(scratch), n, spec.mask_kind,
+                  _hip.ptr(sink), spec.num_v_heads, 1 if spec.out_f32 else 0, hpg, _hip.dtype_code(q.dtype), _hip.stream())
+        return out
+    _hip.call("swl_masked_attn", _hip.ptr(out), _hip.ptr(q), kp, vp, _hip.ptr(block_table), _hip.ptr(tok_seq),
+              _hip.ptr(tok_pos), 0, 0, 0, n, spec.num_q_heads, spec.num_kv_heads, spec.head_dim, spec.value_dim, q.stride(0),
+              spec.window, float(spec.scale), float(spec.softcap), block_table.shape[1], pool.shape[1], spec.mask_kind,
+              _hip.ptr(sink), spec.num_v_heads, 1 if spec.out_f32 else 0, _hip.dtype_code3(q.dtype), _hip.stream())
+    return out
