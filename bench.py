@@ -96,8 +96,11 @@ def parse_args():
     ap.add_argument("--no-reference", action="store_true", help="skip the reference-Triton child run")
     ap.add_argument("--compare-designs", action="store_true",
                     help="instead of the headline workload: prefill and decode throughput of the other designs (Kekapel, "
-                         "Lorulix) beside LLaMA at equal layer sizes (random weights), one JSON line with all")
-    ap.add_argument("--compare", default="llama,kekapel,lorulix", help="designs that --compare-designs runs (comma list)")
+                         "Lorulix, Rosilix) beside LLaMA at equal layer sizes (random weights), one JSON line with all")
+    ap.add_argument("--compare", default="llama,kekapel,lorulix,rosilix",
+                    help="designs that --compare-designs runs (comma list)")
+    ap.add_argument("--compare-kv-rank", type=int, default=512,
+                    help="latent size of Rosilix's latent attention layers in --compare-designs")
     ap.add_argument("--compare-sizes", default="small,medium", help="comma list out of " + ",".join(COMPARE_SIZES))
     return ap.parse_args()
 
@@ -112,7 +115,7 @@ COMPARE_SIZES = {
 }
 
 
-def _compare_configs(sz, positions):
+def _compare_configs(sz, positions, kv_rank=512):
     llama = dict(model_type="llama", hidden_act="silu", rms_norm_eps=1e-5, rope_scaling=None, tie_word_embeddings=False,
                  num_hidden_layers=sz["layers"], hidden_size=sz["heads"] * sz["dim"], num_attention_heads=sz["heads"],
                  num_key_value_heads=sz["kv_heads"], intermediate_size=sz["ff"], vocab_size=sz["vocab"],
@@ -141,7 +144,26 @@ def _compare_configs(sz, positions):
         llayers.append(dict(type="delta" if kind == 1 else "attention", mixer=mixer, mlp=(lmoe if i % 2 else ldense)))
     lorulix = dict(architecture="Lorulix", canon=dict(taps=3), layers=llayers, max_positions=positions,
                    norm=dict(eps=1e-6), vocab=sz["vocab"], width=sz["width"])
-    return llama, kekapel, lorulix
+    # Rosilix at the same sizes: latent attention with a cache of its own / differential attention twice / latent attention
+    # on the first one's cache, in turn. The differential heads hold two maps of dim / 2 (the same query and key widths as
+    # the others' heads) over values of dim, in chunks of 1024; the latent layers have heads of dim + dim / 2 rotated and one
+    # cached row of kv_rank + dim / 2 per token. Squared-ReLU feed-forwards of the dense width.
+    half = sz["dim"] // 2
+    lat = dict(heads=sz["heads"], dim=sz["dim"], rot_dim=half, vdim=sz["dim"], kv_rank=kv_rank,
+               rot=dict(base=10000.0, dims=half), scale=(sz["dim"] + half) ** -0.5)
+    dif = dict(heads=sz["heads"], kv_heads=sz["kv_heads"], dim=half, vdim=sz["dim"], diff=0.3, mask=dict(size=1024),
+               rot=dict(base=10000.0, dims=half), scale=half ** -0.5)
+    rlayers = []
+    for i in range(sz["layers"]):
+        kind = i % 4
+        mixer = dict(dif) if kind in (1, 2) else dict(lat)
+        if kind == 3:
+            mixer["kv_from"] = i - 3
+        rlayers.append(dict(type="attention" if kind in (1, 2) else "latent_attention", mixer=mixer,
+                            mlp=dict(kind="dense", ff=sz["ff"])))
+    rosilix = dict(architecture="Rosilix", embedding=dict(scale=1.0), layers=rlayers, max_positions=positions,
+                   norm=dict(eps=1e-6), vocab=sz["vocab"], width=sz["width"])
+    return llama, kekapel, lorulix, rosilix
 
 
 def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx, steps, warmup):
@@ -203,19 +225,22 @@ def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
 
 def run_compare_designs(args):
     """The designs at every requested size -> one JSON-able dict (rates in tokens/s; ratios: Kekapel / LLaMA, Lorulix /
-    Kekapel — the closest existing design: the same worker, stream and expert kernels — and Lorulix / LLaMA)."""
+    Kekapel — the closest existing design: the same worker, stream and expert kernels — Lorulix / LLaMA, and Rosilix over
+    each of the three: Kekapel is its closest, an all-attention design on the same worker and attention kernels)."""
     results = {}
     for name in [s for s in args.compare_sizes.split(",") if s]:
         sz = COMPARE_SIZES[name]
         prompt_len, prompt_batch, decode_batch, decode_ctx = 2048, 4, 32, 1024
-        configs = dict(zip(("llama", "kekapel", "lorulix"), _compare_configs(sz, prompt_len + 256)))
+        configs = dict(zip(("llama", "kekapel", "lorulix", "rosilix"),
+                           _compare_configs(sz, prompt_len + 256, args.compare_kv_rank)))
         rec = {"sizes": sz, "prompt": [prompt_batch, prompt_len], "decode": [decode_batch, decode_ctx]}
         for label in [d for d in args.compare.split(",") if d]:
             rec[label] = _compare_one(configs[label], args.dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
                                       min(args.steps, 32), min(args.warmup, 8))
             print(f"[compare] {name} {label}: {rec[label]}", file=sys.stderr, flush=True)
         for a, b, key in (("kekapel", "llama", ""), ("lorulix", "kekapel", "lorulix_vs_kekapel_"),
-                          ("lorulix", "llama", "lorulix_vs_llama_")):
+                          ("lorulix", "llama", "lorulix_vs_llama_"), ("rosilix", "kekapel", "rosilix_vs_kekapel_"),
+                          ("rosilix", "lorulix", "rosilix_vs_lorulix_"), ("rosilix", "llama", "rosilix_vs_llama_")):
             if a in rec and b in rec:
                 rec[key + "prefill_ratio"] = rec[a]["prefill_tokens_per_s"] / rec[b]["prefill_tokens_per_s"]
                 rec[key + "decode_ratio"] = rec[a]["decode_tokens_per_s"] / rec[b]["decode_tokens_per_s"]

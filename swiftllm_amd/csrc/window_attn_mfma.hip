@@ -25,7 +25,7 @@ constexpr int kWmWaves = 4;
 constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 
 template <typename T, int D, int DV, int HPW, int NW, bool MIX>
-__global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window_attn_mfma_kernel(
+__global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 512) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk,
     const float *__restrict__ rel, int rel_len, int H, int G,
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4) ? 2 : 1) void window
     // Registers allowing (PIPE), the query fragments stay resident and the next page's key fragments are fetched while this
     // page's mix / softmax / value products run; the value fragments of a page are requested before its score products.
     constexpr int KS = D / 16;
-    constexpr bool PIPE = HPW * D <= 512 && HPW * DV <= 512 && (NW == 4 || HPW * (D + DV) <= 512);   // (eight waves: 256 registers each)
+    constexpr bool PIPE = HPW * D <= 576 && HPW * DV <= 512 && (NW == 4 || HPW * (D + DV) <= 512);   // (eight waves: 256 registers each)
     vec4_t<T> qf[PIPE ? HPW : 1][KS], kf[PIPE ? HPW : 1][KS];
     // element offsets inside a page: of each head's key / value slice (wave-uniform, divided once) and of this lane's fragment
     int koff[HPW], voff[HPW];
@@ -338,8 +338,11 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW, MIX>), grid, dim3(NW * 64), MIX ? lds : 0, s, out, q, kc, \
                        vc, bt, ts, tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf, mask_kind,  \
                        sink, GV, out_f32, hpg)
+    // (a wave's accumulators: HPW * DV / 4 registers — variants beyond 128 of them are not compiled for the wide shapes)
 #define SWL_WM_LAUNCH(HPW, NW)                                 \
-    if (talk) {                                                \
+    if constexpr (!MIXOK && HPW * DV > 512) {                  \
+        return SWL_ERR_UNSUPPORTED;                            \
+    } else if (talk) {                                         \
         if constexpr (MIXOK) SWL_WM_LAUNCH1(HPW, NW, true);    \
         else return SWL_ERR_UNSUPPORTED;                       \
     } else SWL_WM_LAUNCH1(HPW, NW, false)
@@ -367,7 +370,8 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
 // (dim, vdim) pairs with a compiled kernel; the first four also with the head-mixing matrix
 #define SWL_WM_SHAPES_MIX(X) X(64, 64) X(128, 128) X(128, 64) X(64, 128)
 #define SWL_WM_SHAPES_PLAIN(X) \
-    X(32, 32) X(32, 64) X(48, 48) X(48, 96) X(64, 32) X(64, 96) X(96, 64) X(96, 96) X(128, 96) X(96, 128) X(160, 128) X(192, 128)
+    X(32, 32) X(32, 64) X(48, 48) X(48, 96) X(64, 32) X(64, 96) X(96, 64) X(96, 96) X(128, 96) X(96, 128) X(160, 128) X(192, 128) \
+    X(288, 256) X(320, 256) X(576, 512)
 
 static int wm_shape_kind(int dim, int vdim) {      // 2: with or without mixing, 1: without only, 0: none
 #define SWL_WM_IS(DD, DDV) if (dim == DD && vdim == DDV) return 2;
@@ -416,6 +420,12 @@ extern "C" int swl_masked_attn_tiles(void *out, const void *q, const void *k_cac
     if (hpg > 32) {
         if (talk) return SWL_ERR_UNSUPPORTED;
         hpg = 32;
+    }
+    // a group asked for by the caller never needs more accumulators than a wave has registers for: wide value heads go to
+    // more, smaller groups
+    if (!talk && heads_per_group > 0) {
+        const int per_wave = vdim >= 512 ? 1 : vdim >= 256 ? 2 : vdim > 64 ? 4 : 8;
+        if (hpg > 4 * per_wave) hpg = 4 * per_wave;
     }
     if (num_tiles == 0) return SWL_OK;
     if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || !tile_row0 || !tile_cnt ||

@@ -56,13 +56,14 @@ class RosilixLatentAttention:
                                  ctx.tok_pos, mx, w.dkv_col, self.eps)
         # q_abs[t, h, :] = W_uk,h^T q_unrotated[t, h, :]  -> the first kv_rank columns of every head of qa
         qn = proj[:, :H * (d + dr)].view(n, H, d + dr)[:, :, :d].transpose(0, 1)        # [H, T, d]
-        qa.view(n, H, r + dr)[:, :, :r].copy_(torch.bmm(qn, w.uk).transpose(0, 1))
+        torch.bmm(qn, w.uk, out=qa.view(n, H, r + dr)[:, :, :r].transpose(0, 1))      # (a strided batched product: no copy)
         if ctx.pool is None:
             att = torch.zeros((n, H * r), dtype=h.dtype, device=h.device)
         else:
             att = masked_attention(qa, ctx.pool, self.pool_slice, ctx.block_table, ctx.tok_seq, ctx.tok_pos, self.spec,
                                    ctx.tiles, self.max_positions)
-        y = torch.bmm(att.view(n, H, r).transpose(0, 1), w.uv_t).transpose(0, 1).reshape(n, H * e)
+        y = torch.empty((n, H * e), dtype=h.dtype, device=h.device)
+        torch.bmm(att.view(n, H, r).transpose(0, 1), w.uv_t, out=y.view(n, H, e).transpose(0, 1))
         head_gate_(y, proj[:, w.gate_col:w.gate_col + H], H, e)
         return _project(y, w.o, self.skinny)
 

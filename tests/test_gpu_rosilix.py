@@ -201,7 +201,8 @@ def test_latent_attention_alone_and_borrowed(H, d, dr, e, r, n):
 
 
 @pytest.mark.parametrize("H,d,dr,e,r,n", [(6, 32, 32, 48, 64, 150), (4, 64, 32, 64, 96, 90), (16, 16, 16, 32, 48, 70),
-                                          (40, 8, 32, 16, 32, 40), (2, 64, 64, 128, 128, 50)])
+                                          (40, 8, 32, 16, 32, 40), (2, 64, 64, 128, 128, 50), (6, 32, 64, 32, 512, 60),
+                                          (3, 16, 32, 48, 256, 45)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_latent_attention_on_the_matrix_cores(H, d, dr, e, r, n, dtype):
     layers = [O.latent_mixer(heads=H, dim=d, rot_dim=dr, vdim=e, kv_rank=r, scale=(d + dr) ** -0.5)]
