@@ -18,7 +18,9 @@
 //   * sink[H]: a learned logit per head that joins the softmax denominator only (no key, no value, not scaled);
 //   * num_v_heads < num_kv_heads: several key heads share one value head (value head = key head % num_v_heads) — two
 //     score maps over the same values, laid out map-major, are 2 G key heads over G value heads;
-//   * out_f32: the result leaves in fp32 (for a combination of maps that cancels).
+//   * out_f32: the result leaves in fp32 (for a combination of maps that cancels);
+//   * without a mixing matrix the heads are independent: more than 32 of them (or more than the accumulators and the LDS of
+//     one workgroup hold) are shared out over blockIdx.y, every workgroup taking a group of consecutive heads.
 #include "swl_common.h"
 
 namespace swl {
@@ -40,7 +42,8 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const float *talk, const float *rel, int rel_len, int H, int G, int d, int dv,
     int64_t q_tok_stride, int window, float scale, float softcap, int max_blocks_per_seq, int64_t block_stride,
-    int mask_kind, const float *sink, int GV, int out_f32) {
+    int mask_kind, const float *sink, int GV, int out_f32, int Hall) {
+    // H: heads of this workgroup, starting at head hb of the token's Hall heads (G: key heads per Hall query heads)
     extern __shared__ float lds[];
     float *qf = lds;                        // [H * d]
     float *tk = qf + H * d;                 // [H * H]
@@ -56,9 +59,13 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
     const int32_t *bt = block_table + static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq;
     const int lo = window <= 0 ? 0 : mask_kind == 1 ? (pos / window) * window : (pos - window + 1 > 0 ? pos - window + 1 : 0);
     const int nkeys = pos - lo + 1;
-    const int rep = H / G;
+    const int rep = Hall / G;
+    const int hb = static_cast<int>(blockIdx.y) * H;
+    if (hb + H > Hall) H = Hall - hb;
+    if (sink) sink += hb;
+    if (rel) rel += static_cast<int64_t>(hb) * rel_len;
 
-    const T *qrow = q + t * q_tok_stride;
+    const T *qrow = q + t * q_tok_stride + static_cast<int64_t>(hb) * d;
     for (int i = tid; i < H * d; i += kWaThreads) qf[i] = to_f(qrow[i]);
     // (no mixing matrix: every head keeps its own scores)
     for (int i = tid; i < H * H; i += kWaThreads) tk[i] = talk ? talk[i] : (i / H == i % H ? 1.f : 0.f);
@@ -89,7 +96,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
             const int g = idx / kWaChunk, j = idx - g * kWaChunk;
             float v = 0.f;
             if (j < cn) {
-                const T *kr = k_cache + kbase[j] * block_stride + (static_cast<int64_t>(g / rep) * kWaBlock + koff[j]) * d;
+                const T *kr = k_cache + kbase[j] * block_stride + (static_cast<int64_t>((hb + g) / rep) * kWaBlock + koff[j]) * d;
                 const float *qh = qf + g * d;
                 float a = 0.f;
                 for (int e = 0; e < d; ++e) a += qh[e] * to_f(kr[e]);
@@ -134,7 +141,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
             const int idx = tid + i * kWaThreads;
             if (idx < H * dv) {
                 const int h = idx / dv, col = idx - h * dv;
-                const int g = (h / rep) % GV;
+                const int g = ((hb + h) / rep) % GV;
                 float a = acc[i] * alpha[h];
                 const float *ph = p + h * kWaChunk;
                 for (int j = 0; j < cn; ++j) {
@@ -161,7 +168,7 @@ __global__ __launch_bounds__(kWaThreads) void window_attn_kernel(
         if (lane == 0) alpha[h] = al / l;
     }
     __syncthreads();
-    const int64_t obase = t * static_cast<int64_t>(H) * dv;
+    const int64_t obase = (t * static_cast<int64_t>(Hall) + hb) * dv;
 #pragma unroll
     for (int i = 0; i < kWaMaxAcc; ++i) {
         if (i >= nacc) break;
@@ -195,17 +202,27 @@ extern "C" int swl_masked_attn(void *out, const void *q, const void *k_cache, co
     if (num_tokens == 0) return SWL_OK;
     if (!out || !q || !k_cache || !v_cache || !block_table || !tok_seq || !tok_pos || (rel && rel_len <= 0))
         return SWL_ERR_BAD_ARG;
-    const size_t lds = swl::wa_lds_bytes(num_q_heads, dim);
-    if (num_tokens > 0x7fffffffLL || num_q_heads > 32 ||
-        static_cast<int64_t>(num_q_heads) * vdim > swl::kWaMaxAcc * swl::kWaThreads || lds > 64 * 1024)
+    // heads per workgroup: all of them when they are mixed, else as many as its accumulators and LDS hold
+    int hpg = num_q_heads;
+    if (!talk) {
+        if (hpg > 32) hpg = 32;
+        while (hpg > 1 && (static_cast<int64_t>(hpg) * vdim > swl::kWaMaxAcc * swl::kWaThreads ||
+                           swl::wa_lds_bytes(hpg, dim) > 64 * 1024))
+            --hpg;
+    }
+    const size_t lds = swl::wa_lds_bytes(hpg, dim);
+    if (num_tokens > 0x7fffffffLL || hpg > 32 ||
+        static_cast<int64_t>(hpg) * vdim > swl::kWaMaxAcc * swl::kWaThreads || lds > 64 * 1024)
         return SWL_ERR_UNSUPPORTED;
+    const unsigned groups = static_cast<unsigned>((num_q_heads + hpg - 1) / hpg);
     SWL_DISPATCH_DTYPE3(dtype, T, {
-        hipLaunchKernelGGL((swl::window_attn_kernel<T>), dim3(static_cast<unsigned>(num_tokens)), dim3(swl::kWaThreads),
+        hipLaunchKernelGGL((swl::window_attn_kernel<T>), dim3(static_cast<unsigned>(num_tokens), groups),
+                           dim3(swl::kWaThreads),
                            lds, static_cast<hipStream_t>(stream), static_cast<T *>(out), static_cast<const T *>(q),
                            static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, tok_seq,
-                           tok_pos, talk, rel, rel_len, num_q_heads, num_kv_heads, dim, vdim, q_tok_stride, window, scale,
+                           tok_pos, talk, rel, rel_len, hpg, num_kv_heads, dim, vdim, q_tok_stride, window, scale,
                            softcap,
-                           max_blocks_per_seq, block_stride, mask_kind, sink, num_v_heads, out_f32);
+                           max_blocks_per_seq, block_stride, mask_kind, sink, num_v_heads, out_f32, num_q_heads);
     });
     return swl::check_launch();
 }
