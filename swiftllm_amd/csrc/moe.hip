@@ -183,6 +183,24 @@ __global__ __launch_bounds__(kMoeThreads) void relu_sq_kernel(T *y, const T *z, 
     y[i] = to_t<T>(v * v);
 }
 
+// the same for 16-bit rows of a multiple of 8 elements on 16-byte boundaries: 8 elements (16 bytes) per lane
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void relu_sq_wide_kernel(T *y, const T *z, int64_t total8, int ff8,
+                                                                   int64_t in_stride) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kMoeThreads + threadIdx.x;
+    if (i >= total8) return;
+    const int64_t r = i / ff8;
+    const int c = static_cast<int>(i - r * ff8) * 8;
+    const vec8_t<T> x = load8(z + r * in_stride + c);
+    vec8_t<T> o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float v = fmaxf(to_f(x[j]), 0.f);
+        o[j] = to_t<T>(v * v);
+    }
+    store8(y + r * static_cast<int64_t>(ff8) * 8 + c, o);
+}
+
 // grid (tokens, ceil(width / 64)): wave w computes output columns c0 + w, c0 + w + 4, ...
 template <typename T>
 __global__ __launch_bounds__(kMoeThreads) void moe_down_combine_kernel(T *out, const T *y, const T *down,
@@ -547,6 +565,15 @@ extern "C" int swl_relu_sq(void *y, const void *z, int64_t num_rows, int32_t ff,
     if (num_rows == 0) return SWL_OK;
     if (!y || !z) return SWL_ERR_BAD_ARG;
     const int64_t total = num_rows * ff;
+    if (dtype != SWL_F32 && ff % 8 == 0 && in_stride % 8 == 0 && swl::aligned16(y) && swl::aligned16(z)) {
+        const int64_t total8 = total / 8, blocks8 = (total8 + swl::kMoeThreads - 1) / swl::kMoeThreads;
+        SWL_DISPATCH_DTYPE(dtype, T, {
+            hipLaunchKernelGGL((swl::relu_sq_wide_kernel<T>), dim3(static_cast<unsigned>(blocks8)), dim3(swl::kMoeThreads),
+                               0, static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(z), total8,
+                               ff / 8, in_stride);
+        });
+        return swl::check_launch();
+    }
     const int64_t blocks = (total + swl::kMoeThreads - 1) / swl::kMoeThreads;
     if (blocks > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
     SWL_DISPATCH_DTYPE3(dtype, T, {
