@@ -506,6 +506,23 @@ def test_other_sizes(tmp_path, dtype, tol):
     assert close(run_in_portions(model, 2, toks, [100, 1]), want, dtype, tol)
 
 
+@pytest.mark.parametrize("dtype,tol", [("float32", F32_TOL), ("bfloat16", BF16_TOL)])
+def test_sizes_that_are_multiples_of_two_only(tmp_path, dtype, tol):
+    """Width, vocabulary, feed-forward, head and latent sizes that are multiples of nothing but 2: no kernel or projection may
+    lean on an alignment that the common sizes happen to have. Chunks of one position: a token sees itself only."""
+    layers = [O.latent_mixer(heads=3, dim=6, rot_dim=10, vdim=14, kv_rank=22, base=33.0),
+              O.diff_mixer(heads=3, kv_heads=1, dim=10, vdim=6, chunk=13, rot_dims=6, diff=0.2),
+              O.diff_mixer(heads=2, kv_heads=2, dim=6, vdim=22, chunk=1, rot_dims=6, diff=0.45),
+              O.latent_mixer(heads=7, dim=10, rot_dim=10, vdim=6, kv_rank=22, base=33.0, kv_from=0)]
+    cfg = O.make_config(layers, width=50, vocab=77, ff=54, embed_scale=7.0, no_mlp=(1,))
+    W = O.make_weights(cfg, seed=9)
+    toks = tokens_for(cfg, 75, 9)
+    want = O.forward(cfg, W, toks)
+    model = make_model(tmp_path / "m", cfg, W, dtype)
+    assert close(model.step([entry(0, toks, 0)]), want, dtype, tol)
+    assert close(run_in_portions(model, 1, toks, [3, 1, 2, 29, 1]), want, dtype, tol)
+
+
 def test_matrix_core_paths_in_the_model(tmp_path):
     """bfloat16 with head sizes the tiled attention serves: a prompt in portions and decoded tokens against the oracle on the
     same (bf16-representable) weights, with the packed decode projections."""
