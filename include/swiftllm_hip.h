@@ -553,7 +553,9 @@ int swl_window_attn_tiles(void *out, const void *q, const void *k_cache, const v
  *                 maps over the same values: lay the maps out map-major, [map][head].
  *   out_f32       1: out is fp32 whatever dtype says of the operands.
  *   heads_per_group (tiles only; 0: all) heads handled by one workgroup when the heads are not mixed: the heads of a tile
- *                 are shared out over ceil(H / heads_per_group) workgroups.
+ *                 are shared out over ceil(H / heads_per_group) workgroups. -1: the rows of a matrix-core tile are sixteen
+ *                 HEADS of one token instead of sixteen tokens (requires num_tiles == num_tokens, i.e. every tile is one
+ *                 token, num_kv_heads == 1, no talk, no rel): the form for decode steps of heads that share one key head.
  * The tiles form serves more (dim, vdim) pairs without a mixing matrix than with one: ask swl_masked_attn_tiles_supported. */
 int swl_masked_attn(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
                     const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, const float *rel, int32_t rel_len,

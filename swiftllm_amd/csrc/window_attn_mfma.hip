@@ -16,6 +16,12 @@
 // sink[H] (a logit per head that joins the denominator only), num_v_heads (value head = key head % num_v_heads: score maps
 // that share their values), out_f32 (fp32 result), and a split of the heads over blockIdx.z (head_groups: every group of
 // heads_per_group heads is a workgroup of its own — many heads over one shared key head, wide value heads).
+//
+// HEADS mode (decode steps of a layer whose heads all read ONE key head, e.g. latent attention): a tile is one token and the
+// sixteen rows of the matrix-core tile are sixteen HEADS of that token instead of sixteen tokens of one head. The page's key
+// and value fragments are then loaded once for sixteen heads and every product row is a real one, where the token-row form
+// spends fifteen of sixteen rows on padding and repeats the page for every head. One wave per workgroup, grid (tokens, key
+// shares, groups of sixteen heads); the softmax statistics stay per row as before.
 #include "swl_common.h"
 
 namespace swl {
@@ -24,7 +30,7 @@ constexpr int kWmThreads = 256;
 constexpr int kWmWaves = 4;
 constexpr int kWmTile = 16;     // queries per tile = keys per page = MFMA edge
 
-template <typename T, int D, int DV, int HPW, int NW, bool MIX>
+template <typename T, int D, int DV, int HPW, int NW, bool MIX, bool HEADS = false>
 __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 512) ? 2 : 1) void window_attn_mfma_kernel(
     T *out, const T *q, const T *k_cache, const T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
     const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt, const float *__restrict__ talk,
@@ -54,10 +60,12 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
     const int32_t *bt = block_table + static_cast<int64_t>(__builtin_amdgcn_readfirstlane(tok_seq[row0])) * max_blocks_per_seq;
     const int rep = H / G;
     // heads of this workgroup: [hbase, hend); wave w owns HPW of them
-    const int hbase = static_cast<int>(blockIdx.z) * hpg, hend = min(H, hbase + hpg);
-    const int h0 = hbase + wave * HPW;
-    const int qpos = p0 + li;                        // this lane's query position (meaningful when li < cnt)
-    const bool qok = li < cnt;
+    // (HEADS: row li is head hbase + li of the tile's one token; the wave's "head" h0 stands for the group)
+    const int hbase = HEADS ? (static_cast<int>(blockIdx.z) * NW + wave) * kWmTile : static_cast<int>(blockIdx.z) * hpg;
+    const int hend = min(H, hbase + (HEADS ? kWmTile : hpg));
+    const int h0 = HEADS ? hbase : hbase + wave * HPW;
+    const int qpos = HEADS ? p0 : p0 + li;           // this lane's query position (meaningful when li < cnt)
+    const bool qok = HEADS ? hbase + li < H : li < cnt;
     // first visible key of this lane's query, and of the tile's first query
     const int qlo = window <= 0 ? 0 : mask_kind == 1 ? (qpos / window) * window : qpos - window + 1;
     const int lo_first = window <= 0 ? 0 : mask_kind == 1 ? (p0 / window) * window : (p0 - window + 1 > 0 ? p0 - window + 1 : 0);
@@ -80,11 +88,12 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
         for (int ct = 0; ct < CT; ++ct) acc[hh][ct] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
     // the query row this lane feeds as B operand of S^T = K Q^T: row li of the tile (rows past cnt: the tile's last row)
-    const T *qrow = q + static_cast<int64_t>(row0 + (qok ? li : cnt - 1)) * q_tok_stride;
+    const T *qrow = HEADS ? q + static_cast<int64_t>(row0) * q_tok_stride + static_cast<int64_t>(qok ? hbase + li : hbase) * D
+                          : q + static_cast<int64_t>(row0 + (qok ? li : cnt - 1)) * q_tok_stride;
     // Registers allowing (PIPE), the query fragments stay resident and the next page's key fragments are fetched while this
     // page's mix / softmax / value products run; the value fragments of a page are requested before its score products.
     constexpr int KS = D / 16;
-    constexpr bool PIPE = HPW * D <= 576 && HPW * DV <= 512 && (NW == 4 || HPW * (D + DV) <= 512);   // (eight waves: 256 registers each)
+    constexpr bool PIPE = HPW * D <= 576 && HPW * DV <= 512 && (NW <= 4 || HPW * (D + DV) <= 512);   // (eight waves: 256 registers each)
     vec4_t<T> qf[PIPE ? HPW : 1][KS], kf[PIPE ? HPW : 1][KS];
     // element offsets inside a page: of each head's key / value slice (wave-uniform, divided once) and of this lane's fragment
     int koff[HPW], voff[HPW];
@@ -109,7 +118,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
         for (int hh = 0; hh < HPW; ++hh) {
             const int g = min(h0 + hh, H - 1);
 #pragma unroll
-            for (int e = 0; e < KS; ++e) load4(qf[hh][e], qrow + g * D + 4 * lq + e * 16);     // B: query li
+            for (int e = 0; e < KS; ++e) load4(qf[hh][e], qrow + (HEADS ? 0 : g * D) + 4 * lq + e * 16);     // B: query li
         }
     }
     int blk_next = kb0 <= kb1 ? __builtin_amdgcn_readfirstlane(bt[kb0]) : 0;
@@ -150,7 +159,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
                     for (int e = 0; e < KS; ++e) st = mfma16(kf[hh][e], qf[hh][e], st);
                 } else {
                     const T *kr = kblk + koff[hh] + lane_k;
-                    const T *qr = qrow + g * D + 4 * lq;
+                    const T *qr = qrow + (HEADS ? 0 : g * D) + 4 * lq;
 #pragma unroll
                     for (int e = 0; e < KS; ++e) {
                         vec4_t<T> a, b;
@@ -260,8 +269,9 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
             float l = lrun[hh];
             l += __shfl_xor(l, 16, 64);
             l += __shfl_xor(l, 32, 64);
+            const int orow = HEADS ? row0 : row0 + li, ohead = HEADS ? (qok ? hbase + li : hbase) : h;
             if (gridDim.y > 1) {    // partial result of this key share: unnormalised O, running maximum, sum
-                const int64_t slot = (static_cast<int64_t>(blockIdx.y) * num_tokens + row0 + li) * H + h;
+                const int64_t slot = (static_cast<int64_t>(blockIdx.y) * num_tokens + orow) * H + ohead;
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct) {
                     float4_t o = acc[hh][ct];
@@ -276,7 +286,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
             }
             float inv = 1.0f / l;
             if (sink) {     // the sink joins the denominator: rebase the row on max(m, sink) (base-2 units)
-                const float sk = sink[h] * kLog2e, big = fmaxf(mrun[hh], sk);
+                const float sk = sink[ohead] * kLog2e, big = fmaxf(mrun[hh], sk);
                 const float a = fast_exp2(mrun[hh] - big);
                 inv = a / (l * a + fast_exp2(sk - big));
             }
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
                 float4_t o = acc[hh][ct];
                 mfma_results_ready<4>(o);
                 if (qok) {
-                    const int64_t at = (static_cast<int64_t>(row0 + li) * H + h) * DV + ct * 16 + 4 * lq;
+                    const int64_t at = (static_cast<int64_t>(orow) * H + ohead) * DV + ct * 16 + 4 * lq;
                     if (out_f32) {
 #pragma unroll
                         for (int r = 0; r < 4; ++r) o[r] *= inv;
@@ -333,7 +343,19 @@ int launch_wm(int hpw, dim3 grid, size_t lds, hipStream_t s, T *out, const T *q,
               const int32_t *bt, const int32_t *ts, const int32_t *tp, const int32_t *r0, const int32_t *cn,
               const float *talk, const float *rel, int rel_len, int H, int G, int64_t qs, int window, float scale,
               float softcap, int mb, int64_t bs,
-              float *po, float *pml, int64_t nt, int nbuf, int mask_kind, const float *sink, int GV, int out_f32, int hpg) {
+              float *po, float *pml, int64_t nt, int nbuf, int mask_kind, const float *sink, int GV, int out_f32, int hpg,
+              bool heads_mode) {
+    if (heads_mode) {       // rows are heads: one wave per workgroup, grid.z = groups of sixteen heads
+        hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, 1, 1, false, true>), grid, dim3(64), 0, s, out, q, kc, vc, bt, ts,
+                           tp, r0, cn, nullptr, nullptr, 0, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf,
+                           mask_kind, sink, GV, out_f32, hpg);
+        if (grid.y > 1) {
+            const int64_t rows = nt * H;
+            hipLaunchKernelGGL((window_attn_combine_kernel<T>), dim3(static_cast<unsigned>(rows)), dim3(DV < 256 ? 64 : 256), 0,
+                               s, out, po, pml, rows, DV, static_cast<int>(grid.y), sink, H, out_f32);
+        }
+        return check_launch();
+    }
 #define SWL_WM_LAUNCH1(HPW, NW, MIX)                                                                                         \
     hipLaunchKernelGGL((window_attn_mfma_kernel<T, D, DV, HPW, NW, MIX>), grid, dim3(NW * 64), MIX ? lds : 0, s, out, q, kc, \
                        vc, bt, ts, tp, r0, cn, talk, rel, rel_len, H, G, qs, window, scale, softcap, mb, bs, po, pml, nt, nbuf, mask_kind,  \
@@ -413,11 +435,15 @@ extern "C" int swl_masked_attn_tiles(void *out, const void *q, const void *k_cac
     if (num_tiles < 0 || window < 0 || key_splits < 1 || key_splits > 64) return SWL_ERR_BAD_ARG;
     if (key_splits > 1 && (!scratch || num_tokens <= 0 || (reinterpret_cast<uintptr_t>(scratch) & 15)))
         return SWL_ERR_BAD_ARG;
-    if (mask_kind < 0 || mask_kind > 1 || heads_per_group < 0) return SWL_ERR_BAD_ARG;
+    if (mask_kind < 0 || mask_kind > 1 || heads_per_group < -1) return SWL_ERR_BAD_ARG;
+    // heads_per_group -1: the rows of a tile are heads (every tile is ONE token, all heads read one key head, no mix, no bias)
+    const bool heads_mode = heads_per_group == -1;
+    if (heads_mode && (talk || rel || num_kv_heads != 1 || num_tiles != num_tokens)) return SWL_ERR_BAD_ARG;
     if (!swl_masked_attn_tiles_supported(num_q_heads, num_kv_heads, num_v_heads, dim, vdim, dtype)) return SWL_ERR_UNSUPPORTED;
     // heads per workgroup: all of them when they are mixed (the mix couples them), else the caller's choice (0: all)
-    int hpg = (talk || heads_per_group == 0) ? num_q_heads : (heads_per_group < num_q_heads ? heads_per_group : num_q_heads);
-    if (hpg > 32) {
+    int hpg = (talk || heads_per_group <= 0) ? num_q_heads : (heads_per_group < num_q_heads ? heads_per_group : num_q_heads);
+    if (heads_mode) hpg = 16;
+    if (hpg > 32 && !heads_mode) {
         if (talk) return SWL_ERR_UNSUPPORTED;
         hpg = 32;
     }
@@ -452,7 +478,7 @@ extern "C" int swl_masked_attn_tiles(void *out, const void *q, const void *k_cac
                                           static_cast<const T *>(k_cache), static_cast<const T *>(v_cache), block_table, \
                                           tok_seq, tok_pos, tile_row0, tile_cnt, talk, rel, rel_len, num_q_heads, num_kv_heads, \
                                           q_tok_stride, window, scale, softcap, max_blocks_per_seq, block_stride, part_o, \
-                                          part_ml, num_tokens, nbuf, mask_kind, sink, num_v_heads, out_f32, hpg);
+                                          part_ml, num_tokens, nbuf, mask_kind, sink, num_v_heads, out_f32, hpg, heads_mode);
 #define SWL_WM_SHAPE_MIX(DD, DDV) SWL_WM_SHAPE_(DD, DDV, true)
 #define SWL_WM_SHAPE_PLAIN(DD, DDV) SWL_WM_SHAPE_(DD, DDV, false)
     SWL_DISPATCH_DTYPE(dtype, T, {

@@ -83,12 +83,13 @@ def _split_scratch(device, floats: int) -> torch.Tensor:
     return buf
 
 
-def choose_key_splits(num_tiles: int, mixer, max_positions: int) -> int:
-    """Workgroups per tile: enough to occupy the chip when a step has few tiles, never more than the pages a tile can see.
-    A function of the tile count and the model only (not of positions), so a captured decode graph stays valid."""
+def choose_key_splits(num_tiles: int, mixer, max_positions: int, slots: int = _NUM_CUS) -> int:
+    """Workgroups per tile: enough to occupy the chip (`slots` workgroups) when a step has few tiles, never more than the
+    pages a tile can see. A function of the tile count and the model only (not of positions), so a captured decode graph
+    stays valid."""
     span = mixer.window if mixer.window > 0 else max_positions
     pages = span // 16 + 2
-    return max(1, min(_NUM_CUS // max(num_tiles, 1), pages // 4, 16))
+    return max(1, min(slots // max(num_tiles, 1), pages // 4, 16))
 
 
 def tiles_supported(mixer, dtype: torch.dtype) -> bool:
@@ -165,6 +166,10 @@ def masked_tiles_supported(spec: AttentionSpec, dtype: torch.dtype) -> bool:
                                                             spec.head_dim, spec.value_dim, _hip.dtype_code(dtype)))
 
 
+# From this many heads over one shared key head on, a step of single tokens runs with the heads on the matrix-core tile's rows
+HEAD_ROWS_MIN_HEADS = 2
+
+
 def choose_heads_per_group(spec: AttentionSpec) -> int:
     """Heads of one workgroup of the matrix-core kernel (four waves): as many per wave as keep a wave's query, key and value
     fragments and accumulators in registers, so that many or wide heads are shared out over several workgroups."""
@@ -193,9 +198,14 @@ def masked_attention(q: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice,
     wide_ok = q.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0 and kp % 8 == 0 and vp % 8 == 0 and pool.shape[1] % 4 == 0
     if tiles is not None and wide_ok and masked_tiles_supported(spec, q.dtype):
         row0, cnt = tiles
-        hpg = choose_heads_per_group(spec)
-        groups = -(-spec.num_q_heads // hpg)
-        splits = choose_key_splits(row0.shape[0] * groups, spec, max_positions)
+        if spec.num_kv_heads == 1 and row0.shape[0] == n and spec.num_q_heads >= HEAD_ROWS_MIN_HEADS:
+            # every tile is one token (a decode step) and all heads read one key head: the tile's rows are the heads
+            hpg, groups = -1, -(-spec.num_q_heads // 16)
+            splits = choose_key_splits(row0.shape[0] * groups, spec, max_positions, slots=4 * _NUM_CUS)   # (one-wave workgroups)
+        else:
+            hpg = choose_heads_per_group(spec)
+            groups = -(-spec.num_q_heads // hpg)
+            splits = choose_key_splits(row0.shape[0] * groups, spec, max_positions)
         scratch = None
         if splits > 1:
             scratch = _split_scratch(q.device, splits * n * spec.num_q_heads * (spec.value_dim + 2))

@@ -539,6 +539,31 @@ def test_matrix_core_paths_in_the_model(tmp_path):
     assert close(run_in_portions(model, 1, toks, [33, 2, 64, 1]), want, "bfloat16", BF16_TOL)
 
 
+def test_decoding_batches_with_heads_on_the_tile_rows(tmp_path):
+    """bfloat16 decode steps of several sequences of unequal length: every tile is one token, and the latent layers (20 and 6
+    heads over one cached row: a full group of sixteen heads and a partial one) run with their heads on the matrix-core
+    tile's rows; with hipGraph replay."""
+    layers = [O.latent_mixer(heads=20, dim=16, rot_dim=32, vdim=16, kv_rank=64),
+              O.diff_mixer(heads=2, kv_heads=1, dim=32, vdim=64, chunk=32, rot_dims=16),
+              O.latent_mixer(heads=6, dim=32, rot_dim=32, vdim=48, kv_rank=64, kv_from=0)]
+    cfg = O.make_config(layers, width=128, vocab=160, ff=128)
+    W = O.make_weights(cfg, seed=12)
+    lens, starts = [150, 61, 97], [100, 3, 48]
+    reqs = [tokens_for(cfg, n, 70 + i) for i, n in enumerate(lens)]
+    wants = [O.forward(cfg, W, t) for t in reqs]
+    model = make_model(tmp_path / "m", cfg, W, "bfloat16", graph=True)
+    got = [[model.step([entry(i, reqs[i][:starts[i]], 0)])] for i in range(3)]
+    at = list(starts)
+    while any(a < n for a, n in zip(at, lens)):
+        live = [i for i in range(3) if at[i] < lens[i]]
+        lg = model.step([entry(i, reqs[i][at[i]:at[i] + 1], at[i]) for i in live]).clone()
+        for k, i in enumerate(live):
+            got[i].append(lg[k:k + 1])
+            at[i] += 1
+    for i in range(3):
+        assert close(torch.cat(got[i]), wants[i], "bfloat16", BF16_TOL), f"request {i}"
+
+
 def test_first_tokens_of_a_sequence(tmp_path, default_case):
     """Sequences of one to four tokens, alone and decoded, in blocks that longer sequences used before."""
     cfg, W, toks, want, _ = default_case
