@@ -313,28 +313,39 @@ __global__ __launch_bounds__(NW * 64, (HPW <= 2 && NW == 4 && HPW * (D + DV) <= 
     }
 }
 
-// out[t][h][:] = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s over the key shares s (a share without keys has l = 0)
+// out[t][h][:] = sum_s e^{m_s - M} O_s / sum_s e^{m_s - M} l_s over the key shares s (a share without keys has l = 0).
+// The first wave evaluates the shares' weights once (one share per lane, at most 64) and leaves them in LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_combine_kernel(T *out, const float *part_o, const float *part_ml,
                                                                   int64_t rows, int dv, int nsplit, const float *sink, int H,
                                                                   int out_f32) {
+    __shared__ float wgt[64];
+    __shared__ float inv_den;
     const int64_t row = blockIdx.x;     // (token, head)
-    float mx = kNegBig;     // (the maxima are in base-2 exponent units)
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part_ml[(s * rows + row) * 2]);
-    float den = 0.f;
-    if (sink) {
-        const float sk = sink[row % H] * 1.4426950408889634f;
-        mx = fmaxf(mx, sk);
-        den = exp2f(sk - mx);
+    if (threadIdx.x < 64) {
+        const int sp = threadIdx.x;
+        const bool live = sp < nsplit;
+        const float m = live ? part_ml[(sp * rows + row) * 2] : kNegBig;     // (the maxima are in base-2 exponent units)
+        const float l = live ? part_ml[(sp * rows + row) * 2 + 1] : 0.f;
+        float mx = wave_allreduce_max(m);
+        float extra = 0.f;
+        if (sink) {
+            const float sk = sink[row % H] * 1.4426950408889634f;
+            mx = fmaxf(mx, sk);
+            extra = exp2f(sk - mx);
+        }
+        const float w = live ? exp2f(m - mx) : 0.f;
+        const float den = wave_allreduce_sum(w * l) + extra;
+        wgt[sp] = w;
+        if (sp == 0) inv_den = 1.0f / den;
     }
-    for (int s = 0; s < nsplit; ++s)
-        den += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_ml[(s * rows + row) * 2 + 1];
+    __syncthreads();
+    const float inv = inv_den;
     for (int c = threadIdx.x; c < dv; c += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < nsplit; ++s)
-            a += exp2f(part_ml[(s * rows + row) * 2] - mx) * part_o[(s * rows + row) * dv + c];
-        if (out_f32) reinterpret_cast<float *>(out)[row * dv + c] = a / den;
-        else out[row * dv + c] = to_t<T>(a / den);
+        for (int s = 0; s < nsplit; ++s) a += wgt[s] * part_o[(s * rows + row) * dv + c];
+        if (out_f32) reinterpret_cast<float *>(out)[row * dv + c] = a * inv;
+        else out[row * dv + c] = to_t<T>(a * inv);
     }
 }
 
