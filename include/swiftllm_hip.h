@@ -615,18 +615,20 @@ int swl_polynorm(void *out, const void *z, float a, float b, float c, float e, f
 int swl_moe_route(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *bias,
                   int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t dtype, swl_stream_t stream);
 int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *expert_idx, int64_t num_tokens,
-                    int32_t width, int32_t ff, int32_t top, float limit, int32_t dtype, swl_stream_t stream);
+                    int32_t width, int32_t ff, int32_t top, float limit, int32_t act, int32_t dtype, swl_stream_t stream);
 /* Large steps (prompt portions): assignments are sorted by expert and every expert's rows go through the library GEMM;
  * swl_glu_clamp: y[r][f] = act of [gate | up] product rows gate_up[r][2 ff]; swl_moe_combine: out[t] = sum_j w[t][j] *
  * rows[where[t * top + j]] (fp32, fixed order). dtype may be SWL_F32. */
 /* Decode-sized steps, 16-bit, on the matrix core: a workgroup per (expert, 64 outputs) loads every weight fragment once and
  * multiplies it with all assignments of the expert (an expert's weights are streamed once per step). glu = 1: out = y[T * top, ff] from x = h[T, width]
- * and w = gate_up; glu = 0: out = rows[T * top, width] (plain products, for swl_moe_combine) from x = y and w = down. */
+ * and w = gate_up; glu = 0: out = rows[T * top, width] (plain products, for swl_moe_combine) from x = y and w = down.
+ * act (swl_moe_gate_up, swl_glu_clamp): 0 the clamped unit min(g, limit) sigmoid(1.702 g) (clamp(u) + 1), 1 the plain gated
+ * unit silu(g) u (limit unused); swl_moe_expert_stationary takes the latter as glu = 3. */
 int swl_moe_expert_stationary_supported(int64_t num_tokens, int32_t width, int32_t ff, int32_t top, int32_t dtype);
 int swl_moe_expert_stationary(void *out, const void *x, const void *w, const int32_t *expert_idx, int64_t num_tokens,
                               int32_t experts, int32_t width, int32_t ff, int32_t top, int32_t glu, float limit,
                               int32_t dtype, swl_stream_t stream);
-int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
+int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t act, int32_t dtype,
                   swl_stream_t stream);
 int swl_moe_combine(void *out, const void *rows, const int64_t *where, const float *expert_w, int64_t num_tokens,
                     int32_t width, int32_t top, int32_t dtype, swl_stream_t stream);
@@ -686,6 +688,62 @@ int swl_delta_rule(float *o, const float *qn, const float *kn, const float *kq, 
                    int32_t num_qk_heads, int32_t dim, int32_t vdim, swl_stream_t stream);
 int swl_gated_head_rmsnorm(void *out, const float *o, const void *gate, int64_t gate_stride, const float *w, float eps,
                            int64_t num_tokens, int32_t num_heads, int32_t vdim, int32_t dtype, swl_stream_t stream);
+
+/* ---- sigmoid router with group-limited choice (csrc/moe.hip) ---------------------------------------------------------------
+ * s = sigmoid(router[experts, width] h) in fp32. Experts are chosen by s + correction (NULL: by s): the experts form
+ * group_count equal groups of neighbours, a group's score is the sum of its two largest choice scores, only experts of the
+ * group_keep best groups are eligible (group_keep = group_count: all), of these the `top` largest. w_out = the chosen
+ * experts' s divided by their sum (+ 1e-20). dtype may be SWL_F32. */
+int swl_moe_route_grouped(int32_t *idx_out, float *w_out, const void *h, const float *router, const float *correction,
+                          int64_t num_tokens, int32_t width, int32_t experts, int32_t top, int32_t group_count,
+                          int32_t group_keep, int32_t dtype, swl_stream_t stream);
+
+/* ---- projections with biases: per-head q/k RMS norm + value blend + KV store (pool layout of swl_qknorm_store_kv) -----------
+ * q_h <- (q_h + q_b) / rms * q_w (in place; q_w[dim] shared by the heads, NULL: no weight), keys likewise into the pool,
+ * v <- v + v_b, then v <- (1 - mix) v + mix v_other[t] when v_other is given; v is written back into the row and into the
+ * pool. Biases fp32 (NULL: none). k_cache NULL: nothing is stored. dtype may be SWL_F32. */
+int swl_qkv_bias_norm_store(void *qkv, const float *q_b, const float *k_b, const float *v_b, const float *q_w,
+                            const float *k_w, const void *v_other, int64_t v_other_stride, float mix, void *k_cache,
+                            void *v_cache, const int32_t *block_table, const int32_t *tok_seq, const int32_t *tok_pos,
+                            int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim,
+                            int64_t tok_stride, int32_t max_blocks_per_seq, int64_t block_stride, float eps, int32_t dtype,
+                            swl_stream_t stream);
+
+/* ---- sigmoid attention over the pool (csrc/sigmoid_attn.hip) ----------------------------------------------------------------
+ * a[g] = sigmoid(scale q_g . k - r1[g] ln(1 + r2[g] (i - j)) + pb[g]) for every key j <= i (inside `window` when > 0), no
+ * normalisation over keys; a'[h] = sum_g talk[h][g] a[g] (talk NULL: a' = a); out[t][h] = sum_j a'[h] v_j[kv head of h].
+ * r1 / r2 (both or neither), pb, talk: fp32, may be NULL. dtype may be SWL_F32. */
+int swl_sigmoid_attn(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                     const int32_t *tok_seq, const int32_t *tok_pos, const float *talk, const float *r1, const float *r2,
+                     const float *pb, int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
+                     int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, int32_t max_blocks_per_seq,
+                     int64_t block_stride, int32_t dtype, swl_stream_t stream);
+
+/* ---- state-space recurrence with a scalar decay per head (csrc/ssd.hip) -----------------------------------------------------
+ * swl_ssd_prep: proj rows [z | x | B | C | dt] (z, x: heads * vdim; B, C: groups * state; dt: heads) -> xbc [T, x | B | C]
+ * fp32 after the causal convolution (conv_w tap-major [taps, channels], bias conv_b) and SiLU; dt [T, heads] =
+ * softplus(raw + dt_bias); decay = exp(-exp(A_log) dt). swl_ssd_scan: y [T, heads * vdim] fp32 and the states
+ * [heads, state, vdim] at s_off inside the slots: S <- decay S + dt B x^T, y = S^T C + dskip x, one portion per
+ * (seq_row0, seq_cnt) entry. swl_gated_group_rmsnorm: g = y * silu(gate); out = g / rms(g over each of `groups` equal
+ * parts of the row) * w[cols]. dtype (prep, norm) may be SWL_F32. */
+int swl_ssd_prep(float *xbc, float *dt, float *decay, const void *proj, int64_t proj_stride, const float *conv_w,
+                 const float *conv_b, const float *a_log, const float *dt_bias, float *state, int64_t slot_stride,
+                 int64_t tail_off, const int32_t *tok_pos, const int32_t *tok_start, const int32_t *tok_state,
+                 const int32_t *tok_seq, int64_t num_tokens, int32_t num_heads, int32_t vdim, int32_t state_dim,
+                 int32_t groups, int32_t taps, int32_t dtype, swl_stream_t stream);
+int swl_ssd_scan(float *y, const float *xbc, const float *dt, const float *decay, const float *dskip, float *state,
+                 int64_t slot_stride, int64_t s_off, const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos,
+                 const int32_t *tok_state, int32_t num_seqs, int32_t num_heads, int32_t vdim, int32_t state_dim,
+                 int32_t groups, swl_stream_t stream);
+int swl_gated_group_rmsnorm(void *out, const float *y, const void *gate, int64_t gate_stride, const float *w, float eps,
+                            int64_t num_tokens, int32_t cols, int32_t groups, int32_t dtype, swl_stream_t stream);
+
+/* ---- fp32 stream of models that norm a sublayer's RESULT only (csrc/rms_stream.hip) -----------------------------------------
+ * y = coef * (a' + b'), a' = a / rms(a) * wa (wa NULL: a itself), b' likewise (b NULL: none); x += y / rms(y) * w1;
+ * out (may be NULL) = x in the compute dtype, or x / rms(x) * w2 when w2 is given. dtype may be SWL_F32. */
+int swl_post_norm_add(float *x, const void *a, const float *wa, const void *b, const float *wb, float coef, const float *w1,
+                      void *out, const float *w2, float eps, int64_t num_rows, int32_t width, int32_t dtype,
+                      swl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -113,9 +113,9 @@ SIGNATURES = {
     "swl_head_gate": [_P, _P, _I64, _I64, _I32, _I32, _I32, _P],
     "swl_polynorm": [_P, _P, _F32, _F32, _F32, _F32, _F32, _I64, _I32, _I32, _P],
     "swl_moe_route": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
-    "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
+    "swl_moe_gate_up": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _I32, _P],
     "swl_moe_expert_stationary": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _F32, _I32, _P],
-    "swl_glu_clamp": [_P, _P, _I64, _I32, _F32, _I32, _P],
+    "swl_glu_clamp": [_P, _P, _I64, _I32, _F32, _I32, _I32, _P],
     "swl_moe_combine": [_P, _P, _P, _P, _I64, _I32, _I32, _I32, _P],
     "swl_moe_down_combine": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _P],
     "swl_moe_route_scores": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _F32, _I32, _P],
@@ -129,6 +129,16 @@ SIGNATURES = {
                        _I32, _I32, _I32, _P],
     "swl_delta_rule": [_P, _P, _P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
     "swl_gated_head_rmsnorm": [_P, _P, _P, _I64, _P, _F32, _I64, _I32, _I32, _I32, _P],
+    "swl_moe_route_grouped": [_P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _P],
+    "swl_qkv_bias_norm_store": [_P, _P, _P, _P, _P, _P, _P, _I64, _F32, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
+                                _I64, _I32, _I64, _F32, _I32, _P],
+    "swl_sigmoid_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _I32,
+                         _I64, _I32, _P],
+    "swl_ssd_prep": [_P, _P, _P, _P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
+                     _I32, _I32, _P],
+    "swl_ssd_scan": [_P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
+    "swl_gated_group_rmsnorm": [_P, _P, _P, _I64, _P, _F32, _I64, _I32, _I32, _I32, _P],
+    "swl_post_norm_add": [_P, _P, _P, _P, _P, _F32, _P, _P, _P, _F32, _I64, _I32, _I32, _P],
 }
 # Entry points that do not follow the "int rc = f(...)" convention.
 _SPECIAL = {

@@ -38,6 +38,8 @@ SOURCES = [
     "rms_stream.hip",
     "delta_rule.hip",
     "rope_kv.hip",
+    "sigmoid_attn.hip",
+    "ssd.hip",
 ]
 # What a model family's worker calls (the shared pieces included): `build(only=MODEL_SOURCES[...])` compiles just these, so
 # that the first use from a fresh checkout does not pay for kernels the model never launches. A later full build compiles
@@ -51,6 +53,8 @@ MODEL_SOURCES = {
                           "rms_stream.hip", "delta_rule.hip"],
     "Rosilix": _SHARED + ["layernorm.hip", "window_attn.hip", "window_attn_mfma.hip", "moe.hip", "rms_stream.hip",
                           "rope_kv.hip"],
+    "Ratilorn": _SHARED + ["layernorm.hip", "qknorm_kv.hip", "window_attn.hip", "window_attn_mfma.hip", "moe.hip",
+                           "rms_stream.hip", "sigmoid_attn.hip", "ssd.hip"],
 }
 HEADERS = ["swl_common.h", "attend_block.h", "conv_tail.h", os.path.join(ROOT, "include", "swiftllm_hip.h")]
 LIB = os.path.join(HERE, "libswiftllm_hip.so")

@@ -8,6 +8,12 @@
 //   swl_moe_down_combine: out[t] = sum_j weight[t][j] * (W_down[e_j] y[t][j]) with fp32 accumulation through the weighted
 //                         sum (fixed order j = 0, 1, ...: the result does not depend on what else is in the batch).
 //
+//   swl_moe_route_grouped: scores s = sigmoid(router h); experts are CHOSEN by s + correction, inside the `keep` best of
+//                         `count` equal groups of neighbouring experts (a group's score: the sum of its two largest choice
+//                         scores); the weights are the chosen experts' s divided by their sum.
+//   act (swl_moe_gate_up, swl_glu_clamp; glu = 3 of swl_moe_expert_stationary): 0 the clamped unit above, 1 the plain gated
+//                         unit y = silu(g) * u.
+//
 // Expert weights are stacked: gate_up [experts, 2 ff, width] (gate rows, then up rows), down [experts, width, ff].
 #include "swl_common.h"
 
@@ -52,6 +58,14 @@ __device__ __forceinline__ float lane_dot2(const T *x, const T *w, int n, int la
     }
     for (int i = lane; i < n; i += 64) a += to_f(x[i]) * to_f(w[i]);
     return a;
+}
+
+// act 0: g' = min(g, limit), u' = clamp(u, +-limit), g' sigmoid(1.702 g') (u' + 1); act 1: silu(g) u
+__device__ __forceinline__ float gated_unit(float g, float u, float limit, int act) {
+    if (act == 1) return g / (1.0f + expf(-g)) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
 }
 
 template <typename T>
@@ -120,11 +134,118 @@ __global__ __launch_bounds__(kMoeThreads) void moe_route_kernel(int32_t *idx_out
     }
 }
 
+// Sigmoid scores with group-limited choice. One workgroup per token; the first wave chooses.
+template <typename T>
+__global__ __launch_bounds__(kMoeThreads) void moe_route_grouped_kernel(int32_t *idx_out, float *w_out, const T *h,
+                                                                        const float *router, const float *correction,
+                                                                        int width, int experts, int top, int count,
+                                                                        int keep) {
+    extern __shared__ float lds[];
+    float *hf = lds;                    // [width]
+    float *score = hf + width;          // [experts] s = sigmoid(logit)
+    float *choice = score + experts;    // [experts] s + correction; -inf once taken or outside the kept groups
+    float *gscore = choice + experts;   // [count]
+    float *gkeep = gscore + count;      // [count] 1 for the groups whose experts may be chosen
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int i = threadIdx.x; i < width; i += kMoeThreads) hf[i] = to_f(h[t * width + i]);
+    __syncthreads();
+    for (int e = wave; e < experts; e += kMoeWaves) {
+        const float *wr = router + static_cast<int64_t>(e) * width;
+        float a = 0.f;
+        for (int i = lane; i < width; i += 64) a += hf[i] * wr[i];
+        a = wave_allreduce_sum(a);
+        if (lane == 0) {
+            const float sc = 1.0f / (1.0f + expf(-a));
+            score[e] = sc;
+            choice[e] = sc + (correction ? correction[e] : 0.f);
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // arg-max over an LDS array of n floats for the whole wave (ties: the lowest index; -inf never wins)
+    auto argmax = [&](const float *v, int n, float &best, int &besti) {
+        best = -INFINITY;
+        besti = 0x7fffffff;
+        for (int e = lane; e < n; e += 64) {
+            if (v[e] > best) {
+                best = v[e];
+                besti = e;
+            }
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            const float ob = __shfl_xor(best, m, 64);
+            const int oi = __shfl_xor(besti, m, 64);
+            if (ob > best || (ob == best && oi < besti)) {
+                best = ob;
+                besti = oi;
+            }
+        }
+    };
+    if (count > 1 && keep < count) {
+        const int per = experts / count;
+        for (int g = lane; g < count; g += 64) {    // a group's score: its two largest choice scores (one, in groups of one)
+            float a = -INFINITY, b = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; ++e) {
+                const float v = choice[e];
+                if (v > a) {
+                    b = a;
+                    a = v;
+                } else if (v > b) {
+                    b = v;
+                }
+            }
+            gscore[g] = per > 1 ? a + b : a;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+        for (int g = lane; g < count; g += 64) gkeep[g] = 0.f;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+        for (int j = 0; j < keep; ++j) {
+            float best;
+            int besti;
+            argmax(gscore, count, best, besti);
+            if (lane == 0 && besti < count) {
+                gscore[besti] = -INFINITY;      // (taken)
+                gkeep[besti] = 1.f;
+            }
+            __builtin_amdgcn_wave_barrier();
+            __threadfence_block();
+        }
+        for (int e = lane; e < experts; e += 64)
+            if (gkeep[e / per] == 0.f) choice[e] = -INFINITY;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    float denom = 0.f;
+    for (int j = 0; j < top; ++j) {
+        float best;
+        int besti;
+        argmax(choice, experts, best, besti);
+        if (besti >= experts) besti = 0;        // (fewer eligible experts than `top`: cannot happen for keep * per >= top)
+        const float sc = score[besti];
+        denom += sc;
+        if (lane == 0) {
+            idx_out[t * top + j] = besti;
+            w_out[t * top + j] = sc;
+            choice[besti] = -INFINITY;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    if (lane == 0) {
+        const float mult = 1.0f / (denom + 1e-20f);
+        for (int j = 0; j < top; ++j) w_out[t * top + j] *= mult;
+    }
+}
+
 // grid (assignments, ceil(ff / 64)): wave w of the workgroup computes ff rows f0 + w, f0 + w + 4, ...
 template <typename T>
 __global__ __launch_bounds__(kMoeThreads) void moe_gate_up_kernel(T *y, const T *h, const T *gate_up,
                                                                   const int32_t *expert_idx, int width, int ff, int top,
-                                                                  float limit) {
+                                                                  float limit, int act) {
     extern __shared__ float lds[];
     float *hf = lds;    // [width]
     const int64_t a = blockIdx.x;           // assignment = token * top + j
@@ -141,12 +262,7 @@ __global__ __launch_bounds__(kMoeThreads) void moe_gate_up_kernel(T *y, const T 
         float g = lane_dot(hf, rg, width, lane), u = lane_dot(hf, ru, width, lane);
         g = wave_allreduce_sum(g);
         u = wave_allreduce_sum(u);
-        if (lane == 0) {
-            g = fminf(g, limit);
-            u = fminf(fmaxf(u, -limit), limit);
-            const float sg = 1.0f / (1.0f + expf(-1.702f * g));
-            y[a * ff + f] = to_t<T>(g * sg * (u + 1.0f));
-        }
+        if (lane == 0) y[a * ff + f] = to_t<T>(gated_unit(g, u, limit, act));
     }
 }
 
@@ -244,7 +360,7 @@ __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T
     // finishes (short reductions and few outputs would otherwise leave most of the chip idle in a decode step).
     // MODE 0: plain product, X rows are assignments; 1: clamped gated unit, X rows are tokens; 2: squared ReLU of the plain
     // product (experts without a gate), X rows are tokens
-    constexpr bool GLU = MODE == 1;
+    constexpr bool GLU = MODE == 1 || MODE == 3;      // (3: the plain gated unit silu(g) u)
     __shared__ int mine[kEsMaxAssign];
     __shared__ int count;
     __shared__ float red[3][2 * kEsTiles][256];
@@ -358,11 +474,7 @@ __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T
                     const int n = n0 + 4 * lq + r;
                     if (n < N) {
                         float v = accg[t][r];
-                        if constexpr (GLU) {
-                            const float g = fminf(v, limit);
-                            const float u = fminf(fmaxf(accu[t][r], -limit), limit);
-                            v = g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
-                        }
+                        if constexpr (GLU) v = gated_unit(v, accu[t][r], limit, MODE == 3 ? 1 : 0);
                         if constexpr (MODE == 2) {
                             v = fmaxf(v, 0.f);
                             v *= v;
@@ -377,15 +489,13 @@ __global__ __launch_bounds__(kMoeThreads, 2) void moe_expert_stationary_kernel(T
 
 // y[r][f] = act(gu[r][f], gu[r][ff + f]) for rows of [gate | up] products that came from a library GEMM
 template <typename T>
-__global__ __launch_bounds__(kMoeThreads) void glu_clamp_kernel(T *y, const T *gu, int64_t total, int ff, float limit) {
+__global__ __launch_bounds__(kMoeThreads) void glu_clamp_kernel(T *y, const T *gu, int64_t total, int ff, float limit,
+                                                                int act) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * kMoeThreads + threadIdx.x;
     if (i >= total) return;
     const int64_t r = i / ff;
     const int f = static_cast<int>(i - r * ff);
-    float g = fminf(to_f(gu[r * 2 * ff + f]), limit);
-    const float u = fminf(fmaxf(to_f(gu[r * 2 * ff + ff + f]), -limit), limit);
-    const float sg = 1.0f / (1.0f + expf(-1.702f * g));
-    y[i] = to_t<T>(g * sg * (u + 1.0f));
+    y[i] = to_t<T>(gated_unit(to_f(gu[r * 2 * ff + f]), to_f(gu[r * 2 * ff + ff + f]), limit, act));
 }
 
 // out[t] = sum_j w[t][j] * rows[where[t * top + j]]  (fp32 sum in the order j = 0, 1, ...)
@@ -438,6 +548,10 @@ extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w
             hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 2>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
                                assignments, K, N, top, limit, ksplit);
+        else if (glu == 3)
+            hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 3>), grid, dim3(64 * nw), lds, s,
+                               static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
+                               assignments, K, N, top, limit, ksplit);
         else
             hipLaunchKernelGGL((swl::moe_expert_stationary_kernel<T, 0>), grid, dim3(64 * nw), lds, s,
                                static_cast<T *>(out), static_cast<const T *>(x), static_cast<const T *>(w), expert_idx,
@@ -446,9 +560,9 @@ extern "C" int swl_moe_expert_stationary(void *out, const void *x, const void *w
     return swl::check_launch();
 }
 
-extern "C" int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t dtype,
-                             swl_stream_t stream) {
-    if (num_rows < 0 || ff <= 0) return SWL_ERR_BAD_ARG;
+extern "C" int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int32_t ff, float limit, int32_t act,
+                             int32_t dtype, swl_stream_t stream) {
+    if (num_rows < 0 || ff <= 0 || act < 0 || act > 1) return SWL_ERR_BAD_ARG;
     if (num_rows == 0) return SWL_OK;
     if (!y || !gate_up) return SWL_ERR_BAD_ARG;
     const int64_t total = num_rows * ff;
@@ -457,7 +571,7 @@ extern "C" int swl_glu_clamp(void *y, const void *gate_up, int64_t num_rows, int
     SWL_DISPATCH_DTYPE3(dtype, T, {
         hipLaunchKernelGGL((swl::glu_clamp_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(swl::kMoeThreads), 0,
                            static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(gate_up), total,
-                           ff, limit);
+                           ff, limit, act);
     });
     return swl::check_launch();
 }
@@ -509,9 +623,9 @@ extern "C" int swl_moe_route_scores(int32_t *idx_out, float *w_out, const void *
 }
 
 extern "C" int swl_moe_gate_up(void *y, const void *h, const void *gate_up, const int32_t *expert_idx,
-                               int64_t num_tokens, int32_t width, int32_t ff, int32_t top, float limit, int32_t dtype,
-                               swl_stream_t stream) {
-    if (num_tokens < 0 || width <= 0 || ff <= 0 || top <= 0) return SWL_ERR_BAD_ARG;
+                               int64_t num_tokens, int32_t width, int32_t ff, int32_t top, float limit, int32_t act,
+                               int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || ff <= 0 || top <= 0 || act < 0 || act > 1) return SWL_ERR_BAD_ARG;
     if (num_tokens == 0) return SWL_OK;
     if (!y || !h || !gate_up || !expert_idx) return SWL_ERR_BAD_ARG;
     const size_t lds = static_cast<size_t>(width) * 4;
@@ -521,7 +635,7 @@ extern "C" int swl_moe_gate_up(void *y, const void *h, const void *gate_up, cons
     SWL_DISPATCH_DTYPE3(dtype, T, {
         hipLaunchKernelGGL((swl::moe_gate_up_kernel<T>), grid, dim3(swl::kMoeThreads), lds,
                            static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(h),
-                           static_cast<const T *>(gate_up), expert_idx, width, ff, top, limit);
+                           static_cast<const T *>(gate_up), expert_idx, width, ff, top, limit, act);
     });
     return swl::check_launch();
 }
@@ -580,6 +694,24 @@ extern "C" int swl_relu_sq(void *y, const void *z, int64_t num_rows, int32_t ff,
         hipLaunchKernelGGL((swl::relu_sq_kernel<T>), dim3(static_cast<unsigned>(blocks)), dim3(swl::kMoeThreads), 0,
                            static_cast<hipStream_t>(stream), static_cast<T *>(y), static_cast<const T *>(z), total, ff,
                            in_stride);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_moe_route_grouped(int32_t *idx_out, float *w_out, const void *h, const float *router,
+                                     const float *correction, int64_t num_tokens, int32_t width, int32_t experts, int32_t top,
+                                     int32_t group_count, int32_t group_keep, int32_t dtype, swl_stream_t stream) {
+    if (num_tokens < 0 || width <= 0 || experts <= 0 || top <= 0 || top > experts) return SWL_ERR_BAD_ARG;
+    if (group_count < 1 || group_keep < 1 || group_keep > group_count || experts % group_count) return SWL_ERR_BAD_ARG;
+    if (static_cast<int64_t>(group_keep) * (experts / group_count) < top) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!idx_out || !w_out || !h || !router) return SWL_ERR_BAD_ARG;
+    const size_t lds = (static_cast<size_t>(width) + 2 * experts + 2 * group_count) * 4;
+    if (num_tokens > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::moe_route_grouped_kernel<T>), dim3(static_cast<unsigned>(num_tokens)),
+                           dim3(swl::kMoeThreads), lds, static_cast<hipStream_t>(stream), idx_out, w_out,
+                           static_cast<const T *>(h), router, correction, width, experts, top, group_count, group_keep);
     });
     return swl::check_launch();
 }

@@ -148,6 +148,60 @@ __global__ __launch_bounds__(kQkThreads) void qknorm_full_store_kv_kernel(
     }
 }
 
+
+// The same store for projections WITH biases and values that may be blended with the values another layer made for the same
+// token. Per token:
+//   q_h <- (q_h + b_q) / rms(q_h + b_q) * w_q     in place, per head (w_q NULL: no weight)
+//   k_g <- (k_g + b_k) / rms(k_g + b_k) * w_k     into the pool
+//   v   <- v + b_v;  v <- (1 - mix) v + mix v_other[t]  (v_other given)   written back into the row AND into the pool
+// so that the row's value columns can serve as v_other of a later layer. Biases and weights are fp32, all sums fp32.
+template <typename T>
+__global__ __launch_bounds__(kQkThreads) void qkv_bias_norm_store_kernel(
+    T *qkv, const float *q_b, const float *k_b, const float *v_b, const float *q_w, const float *k_w, const T *v_other,
+    int64_t v_other_stride, float mix, T *k_cache, T *v_cache, const int32_t *block_table, const int32_t *tok_seq,
+    const int32_t *tok_pos, int H, int G, int d, int dv, int64_t tok_stride, int max_blocks_per_seq, int64_t block_stride,
+    float eps, int store) {
+    const int64_t t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T *row = qkv + t * tok_stride;
+    const int pos = tok_pos[t];
+    int64_t blk = 0;
+    if (store) blk = block_table[static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq + pos / kQkBlock];
+    const int off = pos % kQkBlock;
+    for (int h = wave; h < H + G; h += kQkThreads / 64) {
+        const bool is_q = h < H;
+        if (!is_q && !store) continue;
+        T *src = row + static_cast<int64_t>(h) * d;         // k heads follow the q heads
+        const float *bias = is_q ? (q_b ? q_b + static_cast<int64_t>(h) * d : nullptr)
+                                 : (k_b ? k_b + static_cast<int64_t>(h - H) * d : nullptr);
+        const float *wn = is_q ? q_w : k_w;
+        float ss = 0.f;
+        for (int e = lane; e < d; e += 64) {
+            const float v = to_f(src[e]) + (bias ? bias[e] : 0.f);
+            ss += v * v;
+        }
+        ss = wave_allreduce_sum(ss);
+        const float r = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+        T *dst = is_q ? src : k_cache + blk * block_stride + (static_cast<int64_t>(h - H) * kQkBlock + off) * d;
+        for (int e = lane; e < d; e += 64) {
+            const float v = (to_f(src[e]) + (bias ? bias[e] : 0.f)) * r;
+            dst[e] = to_t<T>(wn ? v * wn[e] : v);
+        }
+    }
+    T *vsrc = row + static_cast<int64_t>(H + G) * d;
+    const T *vo = v_other ? v_other + t * v_other_stride : nullptr;
+    for (int i = threadIdx.x; i < G * dv; i += kQkThreads) {
+        float v = to_f(vsrc[i]) + (v_b ? v_b[i] : 0.f);
+        if (vo) v = (1.0f - mix) * v + mix * to_f(vo[i]);
+        const T vt = to_t<T>(v);
+        vsrc[i] = vt;
+        if (store) {
+            const int g = i / dv, c = i - g * dv;
+            v_cache[blk * block_stride + (static_cast<int64_t>(g) * dv + c) * kQkBlock + off] = vt;     // transposed page
+        }
+    }
+}
+
 } // namespace swl
 
 extern "C" int swl_qknorm_store_kv(void *qkv, const float *q_w, const float *k_w, void *k_cache, void *v_cache,
@@ -194,6 +248,32 @@ extern "C" int swl_qknorm_full_store_kv(void *qkv, const float *q_w, const float
                            static_cast<T *>(k_cache), static_cast<T *>(v_cache), block_table, tok_seq, tok_pos,
                            num_q_heads, num_kv_heads, dim, vdim, tok_stride, max_blocks_per_seq, block_stride, eps,
                            temp_coef, temp_every, store);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_qkv_bias_norm_store(void *qkv, const float *q_b, const float *k_b, const float *v_b, const float *q_w,
+                                       const float *k_w, const void *v_other, int64_t v_other_stride, float mix,
+                                       void *k_cache, void *v_cache, const int32_t *block_table, const int32_t *tok_seq,
+                                       const int32_t *tok_pos, int64_t num_tokens, int32_t num_q_heads,
+                                       int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t tok_stride,
+                                       int32_t max_blocks_per_seq, int64_t block_stride, float eps, int32_t dtype,
+                                       swl_stream_t stream) {
+    if (num_tokens < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || dim <= 0 || vdim <= 0) return SWL_ERR_BAD_ARG;
+    if (num_tokens == 0) return SWL_OK;
+    if (!qkv || !tok_pos) return SWL_ERR_BAD_ARG;
+    const int store = k_cache != nullptr;
+    if (store && (!v_cache || !block_table || !tok_seq)) return SWL_ERR_BAD_ARG;
+    if (tok_stride < static_cast<int64_t>(num_q_heads + num_kv_heads) * dim + static_cast<int64_t>(num_kv_heads) * vdim)
+        return SWL_ERR_BAD_ARG;
+    if (v_other && v_other_stride < static_cast<int64_t>(num_kv_heads) * vdim) return SWL_ERR_BAD_ARG;
+    if (num_tokens > 0x7fffffffLL) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::qkv_bias_norm_store_kernel<T>), dim3(static_cast<unsigned>(num_tokens)),
+                           dim3(swl::kQkThreads), 0, static_cast<hipStream_t>(stream), static_cast<T *>(qkv), q_b, k_b, v_b,
+                           q_w, k_w, static_cast<const T *>(v_other), v_other_stride, mix, static_cast<T *>(k_cache),
+                           static_cast<T *>(v_cache), block_table, tok_seq, tok_pos, num_q_heads, num_kv_heads, dim, vdim,
+                           tok_stride, max_blocks_per_seq, block_stride, eps, store);
     });
     return swl::check_launch();
 }

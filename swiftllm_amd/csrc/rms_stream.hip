@@ -8,6 +8,12 @@
 //       out = x / rms(x) * w2                  the next sublayer's input (or, with row_idx, the norm of selected rows only)
 //     Statistics, gates and the sum are fp32; m, m2, s, r and out are the compute dtype. Weights arrive as the factor itself
 //     (a loader that stores "weight around zero" adds the one).
+//   swl_post_norm_add: the same step for models whose sublayers read the stream itself (norm on the sublayer's RESULT only):
+//       y   = c * (a' + b')      a' = a / rms(a) * wa when wa is given, else a; b' likewise (b optional)
+//       x  += y / rms(y) * w1
+//       out = x in the compute dtype, or x / rms(x) * w2 when w2 is given
+//     Two results normed separately and averaged (mixers side by side: c = 0.5), or two addends summed as they are (routed
+//     experts + a shared expert: c = 1), or one result alone.
 //   swl_causal_conv_state: out[t] = (h[t] if add_input) + sum_j w[j][c] * h[t - taps + 1 + j] per channel (w tap-major) over the tokens of
 //     one sequence, for any cut of the sequence into steps: inputs of earlier steps come from the sequence's state slot,
 //     which keeps the last taps - 1 inputs. The tail is double-buffered: a step reads buffer `parity` and the workgroup of
@@ -66,6 +72,53 @@ __global__ __launch_bounds__(kRsThreads) void gated_add_rmsnorm_kernel(
     for (int i = threadIdx.x; i < width; i += kRsThreads) ss += row[i] * row[i];
     const float rstd = 1.0f / sqrtf(rs_block_sum(ss, red) / static_cast<float>(width) + eps);
     for (int i = threadIdx.x; i < width; i += kRsThreads) out[o * width + i] = to_t<T>(row[i] * rstd * w2[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kRsThreads) void post_norm_add_kernel(float *x, const T *a, const float *wa, const T *b,
+                                                                   const float *wb, float coef, const float *w1, T *out,
+                                                                   const float *w2, float eps, int width) {
+    extern __shared__ float lds[];
+    float *ra = lds, *rb = lds + width, *red = lds + 2 * width;
+    const int64_t t = blockIdx.x;
+    float *xr = x + t * width;
+    float sa = 0.f, sb = 0.f;
+    for (int i = threadIdx.x; i < width; i += kRsThreads) {
+        const float va = to_f(a[t * width + i]);
+        ra[i] = va;
+        sa += va * va;
+        if (b) {
+            const float vb = to_f(b[t * width + i]);
+            rb[i] = vb;
+            sb += vb * vb;
+        }
+    }
+    float na = 1.f, nb = 1.f;
+    if (wa) na = 1.0f / sqrtf(rs_block_sum(sa, red) / static_cast<float>(width) + eps);
+    if (b && wb) nb = 1.0f / sqrtf(rs_block_sum(sb, red) / static_cast<float>(width) + eps);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += kRsThreads) {     // (each thread touches only its own columns of the rows)
+        float y = wa ? ra[i] * na * wa[i] : ra[i];
+        if (b) y += wb ? rb[i] * nb * wb[i] : rb[i];
+        y *= coef;
+        ra[i] = y;
+        ss += y * y;
+    }
+    const float rstd = 1.0f / sqrtf(rs_block_sum(ss, red) / static_cast<float>(width) + eps);
+    float sx = 0.f;
+    for (int i = threadIdx.x; i < width; i += kRsThreads) {
+        const float v = xr[i] + ra[i] * rstd * w1[i];
+        xr[i] = v;
+        ra[i] = v;
+        sx += v * v;
+    }
+    if (!out) return;
+    if (!w2) {
+        for (int i = threadIdx.x; i < width; i += kRsThreads) out[t * width + i] = to_t<T>(ra[i]);
+        return;
+    }
+    const float rx = 1.0f / sqrtf(rs_block_sum(sx, red) / static_cast<float>(width) + eps);
+    for (int i = threadIdx.x; i < width; i += kRsThreads) out[t * width + i] = to_t<T>(ra[i] * rx * w2[i]);
 }
 
 template <typename T>
@@ -140,6 +193,22 @@ extern "C" int swl_causal_conv_state(void *out, int64_t out_stride, const void *
                            dim3(swl::kRsThreads), 0, static_cast<hipStream_t>(stream), static_cast<T *>(out), out_stride,
                            static_cast<const T *>(h), h_stride, w, state, slot_stride, tail_off, tok_pos, tok_start,
                            tok_state, tok_seq, num_tokens, channels, taps, add_input);
+    });
+    return swl::check_launch();
+}
+
+extern "C" int swl_post_norm_add(float *x, const void *a, const float *wa, const void *b, const float *wb, float coef,
+                                 const float *w1, void *out, const float *w2, float eps, int64_t num_rows, int32_t width,
+                                 int32_t dtype, swl_stream_t stream) {
+    if (num_rows < 0 || width <= 0) return SWL_ERR_BAD_ARG;
+    if (num_rows == 0) return SWL_OK;
+    if (!x || !a || !w1 || (wb && !b) || (w2 && !out)) return SWL_ERR_BAD_ARG;
+    const size_t lds = (2 * static_cast<size_t>(width) + swl::kRsThreads / 64) * sizeof(float);
+    if (num_rows > 0x7fffffffLL || lds > 64 * 1024) return SWL_ERR_UNSUPPORTED;
+    SWL_DISPATCH_DTYPE3(dtype, T, {
+        hipLaunchKernelGGL((swl::post_norm_add_kernel<T>), dim3(static_cast<unsigned>(num_rows)), dim3(swl::kRsThreads), lds,
+                           static_cast<hipStream_t>(stream), x, static_cast<const T *>(a), wa, static_cast<const T *>(b), wb,
+                           coef, w1, static_cast<T *>(out), w2, eps, width);
     });
     return swl::check_launch();
 }

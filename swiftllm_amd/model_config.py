@@ -492,3 +492,182 @@ class RosilixModelConfig:
     def load_from_model_path(model_path: str) -> "RosilixModelConfig":
         with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
             return RosilixModelConfig(json.load(f))
+
+
+# ---- Ratilorn --------------------------------------------------------------------------------------------------------------
+class RatilornAttentionConfig:
+    """Attention with biased projections. `sigmoid` = True: keys and queries of unit RMS per head, every visible key weighted by
+    a sigmoid of its score minus a logarithmic distance term, the heads' weights mixed afterwards, values optionally blended
+    with those of the first such layer (`v_mix`). `sigmoid` = False: softmax attention with a weighted q/k norm and no
+    positional term at all."""
+
+    def __init__(self, mixer: dict, sigmoid: bool):
+        self.kind = "sigmoid_attention" if sigmoid else "attention"
+        self.sigmoid = sigmoid
+        self.num_q_heads = int(mixer["heads"])
+        self.num_kv_heads = int(mixer.get("kv_heads", self.num_q_heads))
+        self.head_dim = int(mixer["dim"])
+        self.value_dim = int(mixer.get("vdim", self.head_dim))
+        self.scale = float(mixer["scale"])
+        self.v_mix = bool(mixer.get("v_mix", False)) if sigmoid else False
+        self.softcap = 0.0
+        self.window = 0         # every earlier key is visible
+        if self.num_q_heads % self.num_kv_heads:
+            raise ValueError(f"heads ({self.num_q_heads}) must be a multiple of kv_heads ({self.num_kv_heads})")
+
+    @property
+    def q_size(self) -> int:
+        return self.num_q_heads * self.head_dim
+
+    @property
+    def k_size(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.num_kv_heads * self.value_dim
+
+    @property
+    def o_size(self) -> int:
+        return self.num_q_heads * self.value_dim
+
+
+class StateSpaceConfig:
+    """A state-space recurrence with a scalar decay per head: `heads` heads of `vdim` inputs, a state [state, vdim] per head,
+    B and C shared by the heads of each of `groups` groups, a causal convolution of `conv` taps on x | B | C, and a gated RMS
+    norm of the result in `norm_groups` equal parts."""
+    kind = "state_space"
+
+    def __init__(self, mixer: dict):
+        self.num_heads = int(mixer["heads"])
+        self.value_dim = int(mixer["vdim"])
+        self.state_dim = int(mixer["state"])
+        self.groups = int(mixer.get("groups", 1))
+        self.conv_taps = int(mixer.get("conv", 1))
+        self.norm_groups = int(mixer.get("norm_groups", 1))
+        if self.groups < 1 or self.num_heads % self.groups:
+            raise ValueError(f"heads ({self.num_heads}) must be a multiple of groups ({self.groups})")
+        if self.conv_taps < 1:
+            raise ValueError(f"conv must be positive, got {self.conv_taps}")
+        if self.norm_groups < 1 or self.inner % self.norm_groups:
+            raise ValueError(f"heads * vdim ({self.inner}) must be a multiple of norm_groups ({self.norm_groups})")
+
+    @property
+    def inner(self) -> int:
+        return self.num_heads * self.value_dim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state_dim
+
+    @property
+    def proj_size(self) -> int:
+        """Rows of the input projection: z | x | B | C | dt."""
+        return self.inner + self.conv_channels + self.num_heads
+
+    @property
+    def state_elems(self) -> int:
+        return self.num_heads * self.state_dim * self.value_dim
+
+
+class RatilornParallelConfig:
+    """Two mixers side by side on the same input: softmax attention (`left`) and a state-space recurrence (`right`); the layer
+    takes half the sum of their separately normed results."""
+    kind = "parallel"
+
+    def __init__(self, mixer: dict):
+        self.left = RatilornAttentionConfig(mixer["left"], sigmoid=False)
+        self.right = StateSpaceConfig(mixer["right"])
+
+
+class RatilornMlpConfig:
+    """`dense`: down(silu(gate h) * up h). `moe`: the same unit as experts behind a sigmoid router with a choice correction and
+    group-limited top-k, plus an optional shared expert."""
+
+    def __init__(self, mlp: dict):
+        self.kind = mlp["kind"]
+        self.shared_ffn_inter_dim = 0
+        if self.kind == "dense":
+            self.ffn_inter_dim = int(mlp["ff"])
+        elif self.kind == "moe":
+            router = mlp["router"]
+            self.ffn_inter_dim = int(mlp["expert"]["ff"])
+            self.num_experts = int(router["experts"])
+            self.top_k = int(router["top"])
+            groups = router.get("groups") or {}
+            self.group_count = int(groups.get("count", 1))
+            self.group_keep = int(groups.get("keep", self.group_count))
+            if mlp.get("shared"):
+                self.shared_ffn_inter_dim = int(mlp["shared"]["ff"])
+            if not 0 < self.top_k <= self.num_experts:
+                raise ValueError(f"router.top ({self.top_k}) must be in 1..experts ({self.num_experts})")
+            if self.group_count < 1 or self.num_experts % self.group_count or not 0 < self.group_keep <= self.group_count:
+                raise ValueError(f"bad router groups {groups!r} for {self.num_experts} experts")
+            if self.group_keep * (self.num_experts // self.group_count) < self.top_k:
+                raise ValueError(f"router groups {groups!r} leave fewer than top ({self.top_k}) experts to choose from")
+        else:
+            raise ValueError(f"unsupported mlp.kind {self.kind!r}")
+
+
+class RatilornLayerConfig:
+    def __init__(self, layer: dict):
+        self.type = layer["type"]
+        if self.type == "attention":
+            self.mixer = RatilornAttentionConfig(layer["mixer"], sigmoid=True)
+        elif self.type == "parallel":
+            self.mixer = RatilornParallelConfig(layer["mixer"])
+        else:
+            raise ValueError(f"unsupported layer type {self.type!r}")
+        self.mlp = RatilornMlpConfig(layer["mlp"]) if layer.get("mlp") else None
+
+    @property
+    def attention(self) -> RatilornAttentionConfig:
+        """The layer's attention (the one whose keys and values the block pool holds)."""
+        return self.mixer if self.type == "attention" else self.mixer.left
+
+
+class RatilornModelConfig:
+    """Ratilorn: a decoder-only model with learned positions and an fp32 stream that every sublayer reads as it is; a
+    sublayer's RESULT is RMS-normed (weight stored around zero) and added. Mixers are sigmoid attention with a logarithmic
+    distance penalty and post-sigmoid head mixing, or softmax attention beside a state-space recurrence; feed-forwards are a
+    SiLU gated unit, dense or as a mixture of experts. The embedding table is the output projection too. Every size and
+    constant is read from config.json; layers may differ from one another."""
+
+    def __init__(self, model_config: dict):
+        if model_config.get("architecture") != "Ratilorn":
+            raise AssertionError(f"unsupported architecture {model_config.get('architecture')!r}")
+        self.vocab_size = int(model_config["vocab"])
+        self.hidden_size = int(model_config["width"])
+        self.max_position_embeddings = int(model_config["max_positions"])
+        self.norm_eps = float(model_config["norm"]["eps"])
+        self.logit_scale = float(model_config.get("logit_scale", 1.0))
+        self.layers = [RatilornLayerConfig(layer) for layer in model_config["layers"]]
+        self.num_layers = len(self.layers)
+        # the layers whose values are blended with those of the first of them
+        self.v_mix_layers = [i for i, l in enumerate(self.layers) if l.type == "attention" and l.mixer.v_mix]
+        for i in self.v_mix_layers[1:]:
+            a, b = self.layers[i].mixer, self.layers[self.v_mix_layers[0]].mixer
+            if a.v_size != b.v_size:
+                raise ValueError(f"layer {i}: v_mix needs values of the size of layer {self.v_mix_layers[0]}'s "
+                                 f"({a.v_size} vs {b.v_size})")
+        attn = [l.attention for l in self.layers]
+        # what the scheduler-facing code reads off any model's configuration
+        self.num_q_heads = max(m.num_q_heads for m in attn)
+        self.num_kv_heads = max(m.num_kv_heads for m in attn)
+        self.head_dim = max(m.head_dim for m in attn)
+
+    @property
+    def has_state(self) -> bool:
+        return any(l.type == "parallel" for l in self.layers)
+
+    def kv_elems_per_token(self) -> int:
+        """K and V elements one token occupies over all layers (every layer has one attention)."""
+        return sum(l.attention.k_size + l.attention.v_size for l in self.layers)
+
+    def get_kvslot_size(self, dtype: torch.dtype = torch.bfloat16) -> int:
+        return max(self.kv_elems_per_token(), 1) * dtype.itemsize
+
+    @staticmethod
+    def load_from_model_path(model_path: str) -> "RatilornModelConfig":
+        with open(os.path.join(model_path, "config.json"), "r", encoding="utf-8") as f:
+            return RatilornModelConfig(json.load(f))

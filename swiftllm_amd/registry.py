@@ -14,6 +14,7 @@ MODELS = {
     "Kekapel": ("swiftllm_amd.model_config:KekapelModelConfig", "swiftllm_amd.worker.kekapel_model:KekapelModel"),
     "Lorulix": ("swiftllm_amd.model_config:LorulixModelConfig", "swiftllm_amd.worker.lorulix_model:LorulixModel"),
     "Rosilix": ("swiftllm_amd.model_config:RosilixModelConfig", "swiftllm_amd.worker.rosilix_model:RosilixModel"),
+    "Ratilorn": ("swiftllm_amd.model_config:RatilornModelConfig", "swiftllm_amd.worker.ratilorn_model:RatilornModel"),
 }
 
 

@@ -109,8 +109,38 @@ def _identity(n: int, device) -> torch.Tensor:
     return t
 
 
+ACT_CLAMPED = 0     # min(g, limit) * sigmoid(1.702 g) * (clamp(u, +-limit) + 1)
+ACT_SILU = 1        # silu(g) * u
+
+
+def gated_unit(gu: torch.Tensor, ff: int, act: int = ACT_SILU, limit: float = 0.0) -> torch.Tensor:
+    """[rows, gate | up] (products of a fused gate/up projection) -> [rows, ff] through the gated unit `act`."""
+    assert gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] == 2 * ff
+    y = torch.empty((gu.shape[0], ff), dtype=gu.dtype, device=gu.device)
+    _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), gu.shape[0], ff, float(limit), int(act),
+              _hip.dtype_code3(gu.dtype), _hip.stream())
+    return y
+
+
+def moe_route_grouped(h: torch.Tensor, router: torch.Tensor, correction: torch.Tensor, top_k: int, group_count: int = 1,
+                      group_keep: int = 1):
+    """-> (expert ids int32 [T, top_k], weights fp32 [T, top_k]). Scores s = sigmoid(router h) in fp32; the experts are chosen
+    by s + correction among the experts of the group_keep best of group_count equal groups (a group's score: its two largest
+    choice scores added); weights = s of the chosen experts over their sum."""
+    _hip.require_gpu_tensor(h, "h")
+    n, width = h.shape
+    experts = router.shape[0]
+    assert h.is_contiguous() and router.dtype == torch.float32 and router.is_contiguous() and router.shape[1] == width
+    assert correction is None or (correction.dtype == torch.float32 and correction.numel() == experts)
+    idx = torch.empty((n, top_k), dtype=torch.int32, device=h.device)
+    wts = torch.empty((n, top_k), dtype=torch.float32, device=h.device)
+    _hip.call("swl_moe_route_grouped", _hip.ptr(idx), _hip.ptr(wts), _hip.ptr(h), _hip.ptr(router), _hip.ptr(correction), n,
+              width, experts, top_k, int(group_count), int(group_keep), _hip.dtype_code3(h.dtype), _hip.stream())
+    return idx, wts
+
+
 def moe_experts_grouped(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                        limit: float) -> torch.Tensor:
+                        limit: float, act: int = ACT_CLAMPED) -> torch.Tensor:
     """The same function as moe_experts for steps with many tokens: assignments sorted by expert (stable), one [rows, width]
     x [width, 2 ff] and one [rows, ff] x [ff, width] library product per expert that received tokens, the activation and
     the weighted combination as kernels. Reads the per-expert counts back to the host (one sync per call)."""
@@ -131,7 +161,7 @@ def moe_experts_grouped(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, g
             torch.mm(xs[off:off + c], gate_up[e].t(), out=gu[off:off + c])
             off += c
     y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
-    _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), n * top_k, ff, float(limit), code, stream)
+    _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), n * top_k, ff, float(limit), int(act), code, stream)
     rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
     off = 0
     for e, c in enumerate(counts):
@@ -145,22 +175,22 @@ def moe_experts_grouped(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, g
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor,
-                limit: float) -> torch.Tensor:
+                limit: float, act: int = ACT_CLAMPED) -> torch.Tensor:
     """-> [T, width]: sum_j wts[t, j] * expert idx[t, j] applied to h[t]. gate_up [experts, 2 ff, width], down
-    [experts, width, ff]."""
+    [experts, width, ff]. act: the experts' gated unit (ACT_CLAMPED with `limit`, or ACT_SILU)."""
     n, width = h.shape
     experts, two_ff, _ = gate_up.shape
     ff, top_k = two_ff // 2, idx.shape[1]
     assert gate_up.is_contiguous() and down.is_contiguous() and down.shape == (experts, width, ff)
     assert gate_up.dtype == down.dtype == h.dtype and idx.dtype == torch.int32 and wts.dtype == torch.float32
     if n * top_k >= GROUPED_MIN_ROWS_PER_EXPERT * experts and not torch.cuda.is_current_stream_capturing():
-        return moe_experts_grouped(h, idx, wts, gate_up, down, limit)
+        return moe_experts_grouped(h, idx, wts, gate_up, down, limit, act)
     code, stream = _hip.dtype_code3(h.dtype), _hip.stream()
     if h.dtype != torch.float32 and _hip.load().swl_moe_expert_stationary_supported(n, width, ff, top_k, code):
         # decode-sized 16-bit step: every expert's weights are read once, whatever the number of tokens that chose it
         y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
         _hip.call("swl_moe_expert_stationary", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, experts,
-                  width, ff, top_k, 1, float(limit), code, stream)
+                  width, ff, top_k, 3 if act == ACT_SILU else 1, float(limit), code, stream)
         rows = torch.empty((n * top_k, width), dtype=h.dtype, device=h.device)
         _hip.call("swl_moe_expert_stationary", _hip.ptr(rows), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), n, experts,
                   width, ff, top_k, 0, float(limit), code, stream)
@@ -170,7 +200,7 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate_up: 
         return out
     y = torch.empty((n * top_k, ff), dtype=h.dtype, device=h.device)
     _hip.call("swl_moe_gate_up", _hip.ptr(y), _hip.ptr(h), _hip.ptr(gate_up), _hip.ptr(idx), n, width, ff, top_k,
-              float(limit), code, stream)
+              float(limit), int(act), code, stream)
     out = torch.empty((n, width), dtype=h.dtype, device=h.device)
     _hip.call("swl_moe_down_combine", _hip.ptr(out), _hip.ptr(y), _hip.ptr(down), _hip.ptr(idx), _hip.ptr(wts), n, width,
               ff, top_k, code, stream)

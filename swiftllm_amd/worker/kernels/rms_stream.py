@@ -34,6 +34,26 @@ def gated_add_rmsnorm(x: torch.Tensor, m: torch.Tensor = None, post: torch.Tenso
     return out
 
 
+def post_norm_add(x: torch.Tensor, a: torch.Tensor, post: torch.Tensor, b: torch.Tensor = None, a_norm: torch.Tensor = None,
+                  b_norm: torch.Tensor = None, coef: float = 1.0, pre: torch.Tensor = None, eps: float = 1e-6,
+                  want_out: bool = True):
+    """In place on the fp32 stream x [T, width], for models whose sublayers read the stream itself:
+        y = coef * (a' + b');  x += y / rms(y) * post
+    with a' = a / rms(a) * a_norm when a_norm is given (else a), b' likewise (b optional). Returns the next sublayer's input
+    in a's dtype: x itself, or x / rms(x) * pre when `pre` is given (None when not wanted)."""
+    _hip.require_gpu_tensor(x, "x")
+    n, width = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous() and a.shape == x.shape and a.is_contiguous()
+    assert b is None or (b.shape == x.shape and b.is_contiguous() and b.dtype == a.dtype)
+    for w in (post, a_norm, b_norm, pre):
+        assert w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == width)
+    out = torch.empty((n, width), dtype=a.dtype, device=x.device) if want_out else None
+    _hip.call("swl_post_norm_add", _hip.ptr(x), _hip.ptr(a), _hip.ptr(a_norm), _hip.ptr(b), _hip.ptr(b_norm), float(coef),
+              _hip.ptr(post), _hip.ptr(out), _hip.ptr(pre) if want_out else 0, float(eps), n, width,
+              _hip.dtype_code3(a.dtype), _hip.stream())
+    return out
+
+
 class StateRef:
     """Where a step's kernels find per-sequence state: the slot pool, and the plan's per-token arrays."""
     __slots__ = ("pool", "tok_pos", "tok_start", "tok_state", "tok_seq", "seq_row0", "seq_cnt")

@@ -64,6 +64,38 @@ def qknorm_full_and_store_kv(q_or_qkv: torch.Tensor, q_norm: torch.Tensor, k_nor
               int(mixer.q_temp_every), _hip.dtype_code3(q_or_qkv.dtype), _hip.stream())
 
 
+def qkv_bias_norm_store(qkv: torch.Tensor, q_b: torch.Tensor, k_b: torch.Tensor, v_b: torch.Tensor, q_norm: torch.Tensor,
+                        k_norm: torch.Tensor, pool: torch.Tensor, pool_slice: PoolSlice, block_table: torch.Tensor,
+                        tok_seq: torch.Tensor, tok_pos: torch.Tensor, mixer, eps: float, v_other: torch.Tensor = None,
+                        mix: float = 0.0):
+    """qkv [T, q | k | v] of one fused projection whose biases (fp32, optional) are still to be added: q heads biased and
+    normed in place (q_norm / k_norm [dim] fp32 weights shared by the heads, None: unit RMS without a weight), k heads biased
+    and normed into the pool, v biased, blended as (1 - mix) v + mix v_other[t] when v_other [T, kv_heads * vdim] (a column
+    slice is fine) is given, and written both back into its columns and into the pool. pool None: no store."""
+    _hip.require_gpu_tensor(qkv, "qkv")
+    assert qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] >= mixer.q_size + mixer.k_size + mixer.v_size
+    for t, size in ((q_b, mixer.q_size), (k_b, mixer.k_size), (v_b, mixer.v_size), (q_norm, mixer.head_dim),
+                    (k_norm, mixer.head_dim)):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == size)
+    assert tok_pos.dtype == torch.int32 and tok_pos.shape[0] == qkv.shape[0]
+    assert v_other is None or (v_other.dtype == qkv.dtype and v_other.stride(1) == 1 and v_other.shape[0] == qkv.shape[0]
+                               and v_other.shape[1] == mixer.v_size)
+    kp = vp = stride = 0
+    if pool is not None:
+        assert pool.is_contiguous() and pool.dtype == qkv.dtype and block_table.is_contiguous()
+        assert tok_seq.dtype == torch.int32 and tok_seq.shape[0] == qkv.shape[0]
+        esize = pool.element_size()
+        kp = pool.data_ptr() + pool_slice.k_offset * esize
+        vp = pool.data_ptr() + pool_slice.v_offset * esize
+        stride = pool.shape[1]
+    _hip.call("swl_qkv_bias_norm_store", _hip.ptr(qkv), _hip.ptr(q_b), _hip.ptr(k_b), _hip.ptr(v_b), _hip.ptr(q_norm),
+              _hip.ptr(k_norm), _hip.ptr(v_other), v_other.stride(0) if v_other is not None else 0, float(mix), kp, vp,
+              _hip.ptr(block_table), _hip.ptr(tok_seq), _hip.ptr(tok_pos), qkv.shape[0], mixer.num_q_heads,
+              mixer.num_kv_heads, mixer.head_dim, mixer.value_dim, qkv.stride(0),
+              block_table.shape[1] if block_table is not None else 0, stride, float(eps), _hip.dtype_code3(qkv.dtype),
+              _hip.stream())
+
+
 # Steps with at least this many tokens go to the matrix-core kernel (tiles of up to 16 queries; a decoded token is a tile of
 # one: the matrix core is mostly padding there, but the kernel reads every page once with wide loads and shares a tile's pages
 # out over several workgroups when there are few tiles).

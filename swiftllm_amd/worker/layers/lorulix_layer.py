@@ -68,7 +68,7 @@ class LorulixFeedForward:
         if mlp.kind == "dense":
             gu = _project(h, w.gate_up, self.skinny)
             y = torch.empty((h.shape[0], mlp.ffn_inter_dim), dtype=h.dtype, device=h.device)
-            _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), h.shape[0], mlp.ffn_inter_dim, float(mlp.limit),
+            _hip.call("swl_glu_clamp", _hip.ptr(y), _hip.ptr(gu), h.shape[0], mlp.ffn_inter_dim, float(mlp.limit), 0,
                       _hip.dtype_code3(h.dtype), _hip.stream())
             return _project(y, w.down, self.skinny), None, None
         idx, wts = moe_route_scores(h, w.router, mlp.top_k, mlp.router_scale)
