@@ -718,6 +718,16 @@ int swl_sigmoid_attn(void *out, const void *q, const void *k_cache, const void *
                      const float *pb, int64_t num_tokens, int32_t num_q_heads, int32_t num_kv_heads, int32_t dim,
                      int32_t vdim, int64_t q_tok_stride, int32_t window, float scale, int32_t max_blocks_per_seq,
                      int64_t block_stride, int32_t dtype, swl_stream_t stream);
+/* The matrix-core form (16-bit storage): tiles of up to 16 consecutive queries of one sequence (tile_row0, tile_cnt) against
+ * 16-key pages; key_splits > 1: every tile's pages are shared out over that many workgroups, whose fp32 partial sums
+ * (scratch: key_splits * num_tokens * heads * vdim floats) a second launch adds up. */
+int swl_sigmoid_attn_tiles_supported(int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int32_t dtype);
+int swl_sigmoid_attn_tiles(void *out, const void *q, const void *k_cache, const void *v_cache, const int32_t *block_table,
+                           const int32_t *tok_seq, const int32_t *tok_pos, const int32_t *tile_row0, const int32_t *tile_cnt,
+                           const float *talk, const float *r1, const float *r2, const float *pb, int32_t num_tiles,
+                           int32_t num_q_heads, int32_t num_kv_heads, int32_t dim, int32_t vdim, int64_t q_tok_stride,
+                           int32_t window, float scale, int32_t max_blocks_per_seq, int64_t block_stride, int32_t key_splits,
+                           float *scratch, int64_t num_tokens, int32_t dtype, swl_stream_t stream);
 
 /* ---- state-space recurrence with a scalar decay per head (csrc/ssd.hip) -----------------------------------------------------
  * swl_ssd_prep: proj rows [z | x | B | C | dt] (z, x: heads * vdim; B, C: groups * state; dt: heads) -> xbc [T, x | B | C]

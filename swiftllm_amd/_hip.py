@@ -134,6 +134,8 @@ SIGNATURES = {
                                 _I64, _I32, _I64, _F32, _I32, _P],
     "swl_sigmoid_attn": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32, _I64, _I32, _F32, _I32,
                          _I64, _I32, _P],
+    "swl_sigmoid_attn_tiles": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I64, _I32,
+                               _F32, _I32, _I64, _I32, _P, _I64, _I32, _P],
     "swl_ssd_prep": [_P, _P, _P, _P, _I64, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I64, _I32, _I32, _I32, _I32,
                      _I32, _I32, _P],
     "swl_ssd_scan": [_P, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P],
@@ -157,6 +159,7 @@ _SPECIAL = {
     "swl_moe_expert_stationary_supported": ([_I64, _I32, _I32, _I32, _I32], _I32),
     "swl_window_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32], _I32),
     "swl_masked_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32, _I32], _I32),
+    "swl_sigmoid_attn_tiles_supported": ([_I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_supported": ([_I32, _I32, _I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_slots_per_layer": ([_I32, _I32, _I32, _I32], _I32),
     "swl_decode_engine_workspace_bytes": ([_I32, _I32, _I32, _I32], ctypes.c_size_t),

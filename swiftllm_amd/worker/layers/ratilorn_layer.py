@@ -23,8 +23,9 @@ class RatilornSigmoidAttention:
     """(q | k | v) projection -> biases, unit q/k per head, value blend, KV store -> sigmoid attention over every earlier key
     with the logarithmic distance penalty and post-sigmoid head mixing -> output projection."""
 
-    def __init__(self, layer_config, weight, eps: float, skinny: bool, pool_slice):
+    def __init__(self, layer_config, weight, eps: float, skinny: bool, pool_slice, max_positions: int):
         self.mixer, self.w, self.eps, self.skinny, self.pool_slice = layer_config.mixer, weight, eps, skinny, pool_slice
+        self.max_positions = max_positions
 
     def forward(self, h: torch.Tensor, ctx: StepContext, share: ValueShare):
         mx, w = self.mixer, self.w
@@ -38,7 +39,7 @@ class RatilornSigmoidAttention:
             attn = torch.zeros((h.shape[0], mx.o_size), dtype=h.dtype, device=h.device)
         else:
             attn = sigmoid_attention(qkv, ctx.pool, self.pool_slice, ctx.block_table, ctx.tok_seq, ctx.tok_pos, mx, w.talk,
-                                     w.r1, w.r2, w.pb, ctx.tiles)
+                                     w.r1, w.r2, w.pb, ctx.tiles, self.max_positions)
         return _project(attn, w.o, self.skinny), None
 
 

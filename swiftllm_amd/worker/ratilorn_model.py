@@ -77,7 +77,7 @@ class RatilornModel(SteppedModel):
         for i, (lcfg, lw) in enumerate(zip(cfg.layers, self.weight.layers)):
             s = _Sublayer()
             if lcfg.type == "attention":
-                s.op = RatilornSigmoidAttention(lcfg, lw, eps, skinny, self.pool_slices[i])
+                s.op = RatilornSigmoidAttention(lcfg, lw, eps, skinny, self.pool_slices[i], cfg.max_position_embeddings)
                 s.a_norm = s.b_norm = None
                 s.coef = 1.0
             else:

@@ -295,3 +295,40 @@ def write_checkpoint(path: str, config: dict, W: dict):
         f.write(head)
         for b in blobs:
             f.write(b)
+
+
+# ---- configurations for the tests ------------------------------------------------------------------------------------------
+def dense_mlp(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe_mlp(ff=24, experts=8, top=2, groups=(4, 2), shared=16):
+    router = {"experts": experts, "top": top}
+    if groups:
+        router["groups"] = {"count": groups[0], "keep": groups[1]}
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": router}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, v_mix=True, scale=None, mlp="dense"):
+    return {"type": "attention", "mlp": dense_mlp() if mlp == "dense" else mlp,
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "v_mix": v_mix,
+                      "scale": scale if scale is not None else dim ** -0.5}}
+
+
+def parallel_layer(heads=4, kv_heads=2, dim=16, vdim=16, s_heads=3, s_vdim=8, state=12, groups=1, conv=3, norm_groups=1,
+                   scale=None, mlp="moe"):
+    return {"type": "parallel", "mlp": moe_mlp() if mlp == "moe" else mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                               "scale": scale if scale is not None else dim ** -0.5},
+                      "right": {"heads": s_heads, "vdim": s_vdim, "state": state, "groups": groups, "conv": conv,
+                                "norm_groups": norm_groups}}}
+
+
+def make_config(layers=None, width=40, vocab=61, max_positions=160, eps=1e-5, logit_scale=0.5):
+    if layers is None:
+        layers = [attention_layer(), parallel_layer(), attention_layer(mlp=moe_mlp()), parallel_layer(mlp=dense_mlp())]
+    return {"architecture": "Ratilorn", "vocab": vocab, "width": width, "max_positions": max_positions,
+            "norm": {"eps": eps}, "logit_scale": logit_scale, "layers": layers}
