@@ -96,8 +96,9 @@ def parse_args():
     ap.add_argument("--no-reference", action="store_true", help="skip the reference-Triton child run")
     ap.add_argument("--compare-designs", action="store_true",
                     help="instead of the headline workload: prefill and decode throughput of the other designs (Kekapel, "
-                         "Lorulix, Rosilix) beside LLaMA at equal layer sizes (random weights), one JSON line with all")
-    ap.add_argument("--compare", default="llama,kekapel,lorulix,rosilix",
+                         "Lorulix, Rosilix, Ratilorn) beside LLaMA at equal layer sizes (random weights), one JSON line "
+                         "with all")
+    ap.add_argument("--compare", default="llama,kekapel,lorulix,rosilix,ratilorn",
                     help="designs that --compare-designs runs (comma list)")
     ap.add_argument("--compare-kv-rank", type=int, default=512,
                     help="latent size of Rosilix's latent attention layers in --compare-designs")
@@ -163,7 +164,21 @@ def _compare_configs(sz, positions, kv_rank=512):
                             mlp=dict(kind="dense", ff=sz["ff"])))
     rosilix = dict(architecture="Rosilix", embedding=dict(scale=1.0), layers=rlayers, max_positions=positions,
                    norm=dict(eps=1e-6), vocab=sz["vocab"], width=sz["width"])
-    return llama, kekapel, lorulix, rosilix
+    # Ratilorn at the same sizes: sigmoid attention (all of them blending their values with the first one's) / two parallel
+    # layers (softmax attention beside a state-space recurrence of the delta layers' width: heads of dim inputs, a state of
+    # dim per head, 4 taps), in turn; the same dense and expert widths as Lorulix, the experts in 4 groups of which 2 are kept
+    sattn = dict(dim=sz["dim"], vdim=sz["dim"], heads=sz["heads"], kv_heads=sz["kv_heads"], scale=sz["dim"] ** -0.5,
+                 v_mix=True)
+    par = dict(left=dict(dim=sz["dim"], vdim=sz["dim"], heads=sz["heads"], kv_heads=sz["kv_heads"], scale=sz["dim"] ** -0.5),
+               right=dict(heads=sz["heads"], vdim=sz["dim"], state=sz["dim"], groups=1, conv=4, norm_groups=1))
+    tmoe = dict(kind="moe", expert=dict(ff=sz["ff"] // 4), router=dict(experts=8, top=2, groups=dict(count=4, keep=2)),
+                shared=dict(ff=sz["ff"] // 4))
+    tdense = dict(kind="dense", ff=sz["ff"])
+    tlayers = [dict(type="parallel" if i % 3 else "attention", mixer=dict(par if i % 3 else sattn),
+                    mlp=(tmoe if i % 2 else tdense)) for i in range(sz["layers"])]
+    ratilorn = dict(architecture="Ratilorn", layers=tlayers, max_positions=positions, norm=dict(eps=1e-6), logit_scale=0.5,
+                    vocab=sz["vocab"], width=sz["width"])
+    return llama, kekapel, lorulix, rosilix, ratilorn
 
 
 def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx, steps, warmup):
@@ -225,13 +240,15 @@ def _compare_one(cfg, dtype, prompt_len, prompt_batch, decode_batch, decode_ctx,
 
 def run_compare_designs(args):
     """The designs at every requested size -> one JSON-able dict (rates in tokens/s; ratios: Kekapel / LLaMA, Lorulix /
-    Kekapel — the closest existing design: the same worker, stream and expert kernels — Lorulix / LLaMA, and Rosilix over
-    each of the three: Kekapel is its closest, an all-attention design on the same worker and attention kernels)."""
+    Kekapel — the closest existing design: the same worker, stream and expert kernels — Lorulix / LLaMA, Rosilix over
+    each of the three: Kekapel is its closest, an all-attention design on the same worker and attention kernels, and Ratilorn
+    over Lorulix — its closest: attention beside a recurrence with state slots, experts with a shared one — Kekapel and
+    LLaMA)."""
     results = {}
     for name in [s for s in args.compare_sizes.split(",") if s]:
         sz = COMPARE_SIZES[name]
         prompt_len, prompt_batch, decode_batch, decode_ctx = 2048, 4, 32, 1024
-        configs = dict(zip(("llama", "kekapel", "lorulix", "rosilix"),
+        configs = dict(zip(("llama", "kekapel", "lorulix", "rosilix", "ratilorn"),
                            _compare_configs(sz, prompt_len + 256, args.compare_kv_rank)))
         rec = {"sizes": sz, "prompt": [prompt_batch, prompt_len], "decode": [decode_batch, decode_ctx]}
         for label in [d for d in args.compare.split(",") if d]:
@@ -240,7 +257,9 @@ def run_compare_designs(args):
             print(f"[compare] {name} {label}: {rec[label]}", file=sys.stderr, flush=True)
         for a, b, key in (("kekapel", "llama", ""), ("lorulix", "kekapel", "lorulix_vs_kekapel_"),
                           ("lorulix", "llama", "lorulix_vs_llama_"), ("rosilix", "kekapel", "rosilix_vs_kekapel_"),
-                          ("rosilix", "lorulix", "rosilix_vs_lorulix_"), ("rosilix", "llama", "rosilix_vs_llama_")):
+                          ("rosilix", "lorulix", "rosilix_vs_lorulix_"), ("rosilix", "llama", "rosilix_vs_llama_"),
+                          ("ratilorn", "lorulix", "ratilorn_vs_lorulix_"), ("ratilorn", "kekapel", "ratilorn_vs_kekapel_"),
+                          ("ratilorn", "llama", "ratilorn_vs_llama_")):
             if a in rec and b in rec:
                 rec[key + "prefill_ratio"] = rec[a]["prefill_tokens_per_s"] / rec[b]["prefill_tokens_per_s"]
                 rec[key + "decode_ratio"] = rec[a]["decode_tokens_per_s"] / rec[b]["decode_tokens_per_s"]

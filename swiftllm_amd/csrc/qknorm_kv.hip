@@ -168,7 +168,47 @@ __global__ __launch_bounds__(kQkThreads) void qkv_bias_norm_store_kernel(
     int64_t blk = 0;
     if (store) blk = block_table[static_cast<int64_t>(tok_seq[t]) * max_blocks_per_seq + pos / kQkBlock];
     const int off = pos % kQkBlock;
-    for (int h = wave; h < H + G; h += kQkThreads / 64) {
+    bool wide = false;
+    if constexpr (sizeof(T) == 2) {
+        // 16-bit heads of 32 / 64 / 128 elements on 16-byte-aligned rows: d / 8 lanes per head move 16 bytes each and several
+        // heads share a wave (the group reduction stays inside d / 8 aligned lanes)
+        wide = (d == 32 || d == 64 || d == 128) && (tok_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
+               (!store || ((reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 && (block_stride & 7) == 0));
+        if (wide) {
+            const int lph = d >> 3;                 // lanes per head: 4, 8 or 16
+            const int hpw = 64 / lph;               // heads per wave and pass
+            const int slot = lane / lph, el = lane - slot * lph;
+            for (int hb = wave * hpw; hb < H + G; hb += (kQkThreads / 64) * hpw) {
+                const int h = hb + slot;
+                const bool live = h < H + G;
+                const bool is_q = h < H;
+                T *src = row + static_cast<int64_t>(live ? h : 0) * d + el * 8;
+                const float *bias = is_q ? q_b : k_b;
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = 0.f;
+                if (live) {
+                    const vec8_t<T> x = load8(src);
+                    const float *bp = bias ? bias + static_cast<int64_t>(is_q ? h : h - H) * d + el * 8 : nullptr;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = to_f(x[j]) + (bp ? bp[j] : 0.f);
+                }
+                float ss = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) ss += v[j] * v[j];
+                ss = lph == 4 ? group_allreduce_sum<4>(ss) : lph == 8 ? group_allreduce_sum<8>(ss) : group_allreduce_sum<16>(ss);
+                const float r = 1.0f / sqrtf(ss / static_cast<float>(d) + eps);
+                if (!live || (!is_q && !store)) continue;
+                const float *wn = is_q ? q_w : k_w;
+                vec8_t<T> o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = to_t<T>(wn ? v[j] * r * wn[el * 8 + j] : v[j] * r);
+                if (is_q) store8(src, o);
+                else store8(k_cache + blk * block_stride + (static_cast<int64_t>(h - H) * kQkBlock + off) * d + el * 8, o);
+            }
+        }
+    }
+    for (int h = wave; h < H + G && !wide; h += kQkThreads / 64) {
         const bool is_q = h < H;
         if (!is_q && !store) continue;
         T *src = row + static_cast<int64_t>(h) * d;         // k heads follow the q heads

@@ -11,7 +11,8 @@
 //   swl_ssd_scan:  one workgroup per (portion, head, share of the columns). The columns of S are independent recurrences:
 //                  a column belongs to L adjacent lanes, each holding state / L of its elements in registers; per token the
 //                  lanes exchange one partial dot product (S^T C) through DPP. B, C, x, dt and the decay of 16 tokens at a
-//                  time are staged in LDS. The token loop is sequential whatever the cut of the sequence into steps: the same
+//                  time are staged in LDS; a wave of loaders stages the next 16 tokens into a second buffer while the others
+//                  walk the current ones. The token loop is sequential whatever the cut of the sequence into steps: the same
 //                  operations in the same order.
 //   swl_gated_group_rmsnorm: out = g / rms(g over a group of columns) * w with g = y * silu(z): gated first, normed
 //                  afterwards, the row in `groups` equal parts.
@@ -69,26 +70,32 @@ __global__ __launch_bounds__(kSsThreads) void ssd_prep_kernel(
     }
 }
 
-template <int MAXDS, int L>
+// LDS rows of B and C are padded by 4 floats per lane slice: the L lanes of a column read L different 16-byte pieces at once,
+// and without the padding slices of 8 / 16 / 32 floats start in the same banks.
+__host__ __device__ inline int ss_row_floats(int N, int L, int ds) { return L * (ds + 4); }
+
+template <int MAXDS, int L, bool EXACT>
 __global__ __launch_bounds__(1024) void ssd_scan_kernel(float *y, const float *xbc, const float *dt, const float *decay,
                                                         const float *dskip, float *state, int64_t slot_stride, int64_t s_off,
                                                         const int32_t *seq_row0, const int32_t *seq_cnt,
                                                         const int32_t *tok_pos, const int32_t *tok_state, int heads, int groups,
-                                                        int N, int P, int cpw, int ds) {
+                                                        int N, int P, int cpw, int ds, int nload) {
+    // nload > 0: the last nload threads of the workgroup only LOAD — they stage chunk c + 1 into the other LDS buffer while
+    // the first threads walk the tokens of chunk c, one barrier per chunk. nload = 0: everybody stages, then walks.
+    // EXACT: ds == MAXDS and L * ds == N (no predicates in the walk).
     extern __shared__ float lds[];
-    float *Bs = lds;                        // [16][N]
-    float *Cs = Bs + kSsChunk * N;          // [16][N]
-    float *xs = Cs + kSsChunk * N;          // [16][cpw]
-    float *dts = xs + kSsChunk * cpw;       // [16]
-    float *das = dts + kSsChunk;            // [16]
+    const int dp = ss_row_floats(N, L, ds);
+    const int buf_floats = kSsChunk * (2 * dp + cpw + 2);
     const int seq = blockIdx.x, h = blockIdx.y;
     const int col0 = blockIdx.z * cpw;
     const int row0 = seq_row0[seq], cnt = seq_cnt[seq];
     const int g = h / (heads / groups);
     const int inner = heads * P, C = inner + 2 * groups * N;
-    const int lc = threadIdx.x / L, l = threadIdx.x % L;
+    const int ncomp = static_cast<int>(blockDim.x) - nload;
+    const bool computes = static_cast<int>(threadIdx.x) < ncomp;
+    const int lc = computes ? threadIdx.x / L : 0, l = threadIdx.x % L;
     const int col = col0 + lc;
-    const bool live = lc < cpw && col < P;       // (threads that pad the workgroup to whole waves own no column)
+    const bool live = computes && lc < cpw && col < P;     // (threads that pad the workgroup to whole waves own no column)
     const int i0 = l * ds;
     float *S = state + static_cast<int64_t>(tok_state[row0] >> 1) * slot_stride + s_off + static_cast<int64_t>(h) * N * P;
     const bool fresh = tok_pos[row0] == 0;      // a sequence starts from the zero state whatever the slot held
@@ -97,39 +104,102 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(float *y, const float *x
     for (int i = 0; i < MAXDS; ++i)
         s[i] = (live && !fresh && i < ds && i0 + i < N) ? S[static_cast<int64_t>(i0 + i) * P + col] : 0.f;
     const float dh = dskip[h];
+    const bool quads = EXACT || (ds & 3) == 0;  // 16-byte LDS reads
 
-    for (int c0 = 0; c0 < cnt; c0 += kSsChunk) {
+    // Stage the chunk at c0 into `buf` with threads sid, sid + sn, ...: all of a thread's loads are issued before the first
+    // one is waited for — one memory round trip per chunk.
+    auto stage = [&](int c0, float *buf, int sid, int sn) {
         const int cn = min(kSsChunk, cnt - c0);
-        __syncthreads();    // the previous chunk has been consumed
-        for (int i = threadIdx.x; i < cn * N; i += blockDim.x) {
-            const int j = i / N, n = i - j * N;
-            const float *src = xbc + static_cast<int64_t>(row0 + c0 + j) * C + inner + g * N + n;
-            Bs[j * N + n] = src[0];
-            Cs[j * N + n] = src[groups * N];
+        float *Bs = buf, *Cs = Bs + kSsChunk * dp, *xs = Cs + kSsChunk * dp, *dts = xs + kSsChunk * cpw, *das = dts + kSsChunk;
+        for (int n = sid; n < N; n += sn) {
+            float tb[kSsChunk], tc[kSsChunk];
+            const float *src = xbc + static_cast<int64_t>(row0 + c0) * C + inner + g * N + n;
+#pragma unroll
+            for (int j = 0; j < kSsChunk; ++j) {
+                const int64_t jj = min(j, cn - 1);      // (rows past the chunk's end re-read its last row: never used)
+                tb[j] = src[jj * C];
+                tc[j] = src[jj * C + groups * N];
+            }
+            const int at = n + 4 * (n / ds);
+#pragma unroll
+            for (int j = 0; j < kSsChunk; ++j) {
+                Bs[j * dp + at] = tb[j];
+                Cs[j * dp + at] = tc[j];
+            }
         }
-        for (int i = threadIdx.x; i < cn * cpw; i += blockDim.x) {
-            const int j = i / cpw, e = i - j * cpw;
-            xs[j * cpw + e] = col0 + e < P ? xbc[static_cast<int64_t>(row0 + c0 + j) * C + h * P + col0 + e] : 0.f;
+        for (int e = sid; e < cpw; e += sn) {
+            float tv[kSsChunk];
+            const float *src = xbc + static_cast<int64_t>(row0 + c0) * C + h * P + min(col0 + e, P - 1);
+#pragma unroll
+            for (int j = 0; j < kSsChunk; ++j) tv[j] = src[static_cast<int64_t>(min(j, cn - 1)) * C];
+#pragma unroll
+            for (int j = 0; j < kSsChunk; ++j) xs[j * cpw + e] = tv[j];
         }
-        for (int j = threadIdx.x; j < cn; j += blockDim.x) {
+        for (int j = sid; j < cn; j += sn) {
             dts[j] = dt[static_cast<int64_t>(row0 + c0 + j) * heads + h];
             das[j] = decay[static_cast<int64_t>(row0 + c0 + j) * heads + h];
         }
-        __syncthreads();
+    };
+
+    // Walk the tokens of the chunk at c0 (staged in `buf`): the sequential part.
+    auto walk = [&](int c0, const float *buf) {
+        const int cn = min(kSsChunk, cnt - c0);
+        const float *Bs = buf, *Cs = Bs + kSsChunk * dp, *xs = Cs + kSsChunk * dp, *dts = xs + kSsChunk * cpw;
+        const float *das = dts + kSsChunk;
+#pragma unroll 2
         for (int j = 0; j < cn; ++j) {
             const float xv = xs[j * cpw + (lc < cpw ? lc : 0)];
             const float dA = das[j], dtx = dts[j] * xv;
-            const float *bj = Bs + j * N + i0, *cj = Cs + j * N + i0;
+            const float *bj = Bs + j * dp + l * (ds + 4), *cj = Cs + j * dp + l * (ds + 4);
+            float br[MAXDS], cr[MAXDS];
+            if (quads) {
+#pragma unroll
+                for (int i = 0; i < MAXDS; i += 4) {
+                    if (EXACT || i < ds) {
+                        const float4_t b4 = *reinterpret_cast<const float4_t *>(bj + i);
+                        const float4_t c4 = *reinterpret_cast<const float4_t *>(cj + i);
+#pragma unroll
+                        for (int c = 0; c < 4; ++c) {
+                            br[i + c] = b4[c];
+                            cr[i + c] = c4[c];
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < MAXDS; ++i) {
+                    br[i] = i < ds ? bj[i] : 0.f;
+                    cr[i] = i < ds ? cj[i] : 0.f;
+                }
+            }
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < MAXDS; ++i) {
-                if (i < ds && i0 + i < N) {
-                    s[i] = fmaf(bj[i], dtx, s[i] * dA);
-                    acc = fmaf(s[i], cj[i], acc);
+                if (EXACT || (i < ds && i0 + i < N)) {
+                    s[i] = fmaf(br[i], dtx, s[i] * dA);
+                    acc = fmaf(s[i], cr[i], acc);
                 }
             }
             acc = group_allreduce_sum<L>(acc);
             if (l == 0 && live) y[static_cast<int64_t>(row0 + c0 + j) * inner + h * P + col] = fmaf(dh, xv, acc);
+        }
+    };
+
+    if (nload > 0) {
+        if (!computes) stage(0, lds, static_cast<int>(threadIdx.x) - ncomp, nload);
+        __syncthreads();
+        int c = 0;
+        for (int c0 = 0; c0 < cnt; c0 += kSsChunk, ++c) {
+            if (computes) walk(c0, lds + (c & 1) * buf_floats);
+            else if (c0 + kSsChunk < cnt) stage(c0 + kSsChunk, lds + ((c + 1) & 1) * buf_floats, static_cast<int>(threadIdx.x) - ncomp, nload);
+            __syncthreads();    // chunk c has been walked and chunk c + 1 is in place
+        }
+    } else {
+        for (int c0 = 0; c0 < cnt; c0 += kSsChunk) {
+            __syncthreads();    // the previous chunk has been consumed
+            stage(c0, lds, threadIdx.x, blockDim.x);
+            __syncthreads();
+            walk(c0, lds);
         }
     }
     if (!live) return;
@@ -170,16 +240,20 @@ template <int L>
 int launch_ssd(int ds, dim3 grid, dim3 block, size_t lds, hipStream_t s, float *y, const float *xbc, const float *dt,
                const float *decay, const float *dskip, float *state, int64_t slot_stride, int64_t s_off,
                const int32_t *seq_row0, const int32_t *seq_cnt, const int32_t *tok_pos, const int32_t *tok_state, int heads,
-               int groups, int N, int P, int cpw) {
-#define SWL_SS_LAUNCH(M)                                                                                                   \
-    hipLaunchKernelGGL((ssd_scan_kernel<M, L>), grid, block, lds, s, y, xbc, dt, decay, dskip, state, slot_stride, s_off, \
-                       seq_row0, seq_cnt, tok_pos, tok_state, heads, groups, N, P, cpw, ds)
-    if (ds <= 8) SWL_SS_LAUNCH(8);
-    else if (ds <= 16) SWL_SS_LAUNCH(16);
-    else if (ds <= 32) SWL_SS_LAUNCH(32);
-    else if (ds <= 64) SWL_SS_LAUNCH(64);
+               int groups, int N, int P, int cpw, int nload) {
+#define SWL_SS_LAUNCH1(M, X)                                                                                                  \
+    hipLaunchKernelGGL((ssd_scan_kernel<M, L, X>), grid, block, lds, s, y, xbc, dt, decay, dskip, state, slot_stride, s_off, \
+                       seq_row0, seq_cnt, tok_pos, tok_state, heads, groups, N, P, cpw, ds, nload)
+#define SWL_SS_LAUNCH(M)                                    \
+    if (ds == M && L * ds == N) SWL_SS_LAUNCH1(M, true);    \
+    else SWL_SS_LAUNCH1(M, false)
+    if (ds <= 8) { SWL_SS_LAUNCH(8); }
+    else if (ds <= 16) { SWL_SS_LAUNCH(16); }
+    else if (ds <= 32) { SWL_SS_LAUNCH(32); }
+    else if (ds <= 64) { SWL_SS_LAUNCH(64); }
     else return SWL_ERR_UNSUPPORTED;
 #undef SWL_SS_LAUNCH
+#undef SWL_SS_LAUNCH1
     return check_launch();
 }
 
@@ -218,23 +292,27 @@ extern "C" int swl_ssd_scan(float *y, const float *xbc, const float *dt, const f
     if (!y || !xbc || !dt || !decay || !dskip || !state || !seq_row0 || !seq_cnt || !tok_pos || !tok_state)
         return SWL_ERR_BAD_ARG;
     if (num_heads > 65535) return SWL_ERR_UNSUPPORTED;
-    // lanes per column: as many (a power of two, at most 16) as keep at least 8 state elements per lane
+    // lanes per column: as many (a power of two, at most 16) as keep at least 16 state elements per lane
     int L = 16;
-    while (L > 1 && (state_dim + L - 1) / L < 8) L >>= 1;
+    while (L > 1 && (state_dim + L - 1) / L < 16) L >>= 1;
     const int ds = (state_dim + L - 1) / L;
     // columns per workgroup: all of them when there are (portion, head) pairs enough to fill the chip; a long prompt alone
     // is a sequential walk, so its columns are shared out over more workgroups (down to 16 columns each)
-    int cpw = vdim < 1024 / L ? vdim : 1024 / L;
+    int cpw = vdim < 960 / L ? vdim : 960 / L;
     while (static_cast<int64_t>(num_seqs) * num_heads * ((vdim + cpw - 1) / cpw) < 512 && cpw % 2 == 0 && cpw > 16) cpw /= 2;
     const unsigned shares = static_cast<unsigned>((vdim + cpw - 1) / cpw);
-    const size_t lds = (static_cast<size_t>(swl::kSsChunk) * (2 * state_dim + cpw + 2)) * sizeof(float);
-    if (lds > 64 * 1024 || shares > 65535) return SWL_ERR_UNSUPPORTED;
+    const size_t one = (static_cast<size_t>(swl::kSsChunk) * (2 * swl::ss_row_floats(state_dim, L, ds) + cpw + 2)) * sizeof(float);
+    if (one > 64 * 1024 || shares > 65535) return SWL_ERR_UNSUPPORTED;
+    const int ncomp = ((cpw * L + 63) / 64) * 64;
+    // a wave of loaders and a second LDS buffer when both fit
+    const int nload = (ncomp + 64 <= 1024 && 2 * one <= 64 * 1024) ? 64 : 0;
+    const size_t lds = nload ? 2 * one : one;
     const dim3 grid(static_cast<unsigned>(num_seqs), static_cast<unsigned>(num_heads), shares);
-    const dim3 block(static_cast<unsigned>(((cpw * L + 63) / 64) * 64));
+    const dim3 block(static_cast<unsigned>(ncomp + nload));
     hipStream_t s = static_cast<hipStream_t>(stream);
 #define SWL_SS_L(LL)                                                                                                          \
     case LL: return swl::launch_ssd<LL>(ds, grid, block, lds, s, y, xbc, dt, decay, dskip, state, slot_stride, s_off, seq_row0, \
-                                        seq_cnt, tok_pos, tok_state, num_heads, groups, state_dim, vdim, cpw)
+                                        seq_cnt, tok_pos, tok_state, num_heads, groups, state_dim, vdim, cpw, nload)
     switch (L) {
         SWL_SS_L(1);
         SWL_SS_L(2);

@@ -681,3 +681,51 @@ def test_greedy_generation_through_the_engine(tmp_path, default_case):
     torch.cuda.empty_cache()
     for g, p, n in zip(got, prompts, outs):
         assert g == oracle(p, n)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_runner_replays_a_mixed_schedule(tmp_path, dtype):
+    """bin/trace_run as a user starts it: five requests through four block-table rows and state slots and a pool of 20 blocks,
+    portions beside decoded tokens, a request that sits steps out, finished requests whose blocks and slot the next one takes."""
+    import json
+    import os
+    import subprocess
+    import sys
+    import numpy as np
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = varied_config()
+    W = O.random_weights(cfg, seed=13)
+    path = str(tmp_path / "m")
+    O.write_checkpoint(path, cfg, W)
+    lens = {"a": 70, "b": 5, "c": 40, "d": 1, "e": 33}
+    reqs = {k: tokens_for(cfg, n, 90 + i) for i, (k, n) in enumerate(lens.items())}
+    schedule = [[("a", 30), ("b", 2), ("c", 17)], [("a", 1), ("b", 1), ("d", 1)], [("a", 2), ("c", 1), ("b", 2)],
+                [("e", 16), ("a", 20)], [("e", 1), ("c", 22)], [("a", 17), ("e", 16)]]
+    at = {k: 0 for k in lens}
+    lines, asked = [], []
+    for n, step in enumerate(schedule):
+        entries, end = [], []
+        for k, c in step:
+            want = list(range(c))[-3:]       # the last three places of every portion
+            entries.append({"id": k, "tokens": reqs[k][at[k]:at[k] + c], "want": want})
+            asked += [(n, k, at[k] + w) for w in want]
+            at[k] += c
+            if at[k] == lens[k]:
+                end.append(k)
+        lines.append(json.dumps({"step": n, "entries": entries, "end": end}))
+    assert at == lens
+    out = tmp_path / "out"
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", dtype, "--out",
+                        str(out), "--max-tokens", "320"], input="\n".join(lines) + "\n", capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {n}" for n in range(len(schedule))]
+    wants = {k: O.forward(f64(W), cfg, t)[0] for k, t in reqs.items()}
+    got, want = [], []
+    for n in range(len(schedule)):
+        rows = [(k, p) for m, k, p in asked if m == n]
+        got.append(torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(len(rows), cfg["vocab"])))
+        want.append(torch.stack([wants[k][p] for k, p in rows]))
+        if dtype == "float32":
+            assert close(got[-1], want[-1], dtype), f"step {n}"
+    assert close(torch.cat(got), torch.cat(want), dtype)
