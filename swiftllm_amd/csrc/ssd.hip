@@ -46,11 +46,15 @@ __global__ __launch_bounds__(kSsThreads) void ssd_prep_kernel(
 #pragma unroll
                 for (int j = 0; j < 8; ++j) cur[j] = to_f(x[j]);
                 tail.conv8(conv_in, proj_stride, conv_w, c, cur, a);
+                float o[8];
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const float v = a[j] + conv_b[c + j];
-                    xbc[t * C + c + j] = v * ss_sigmoid(v);
+                    o[j] = v * ss_sigmoid(v);
                 }
+                float *dst = xbc + t * C + c;       // (C and c are multiples of 8: 32-byte aligned)
+                *reinterpret_cast<float4_t *>(dst) = float4_t{o[0], o[1], o[2], o[3]};
+                *reinterpret_cast<float4_t *>(dst + 4) = float4_t{o[4], o[5], o[6], o[7]};
                 tail.save8(conv_in, proj_stride, c, cur);
             }
         }
