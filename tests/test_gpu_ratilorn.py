@@ -183,13 +183,14 @@ def _attention_weights(H, G, d, e, width, seed, sigmoid):
     return mx, O.random_weights(cfg, seed)
 
 
-def _run_attention(mx, W, p, h, v_other, lam, dtype, sigmoid, portions_of, tiled):
+def _run_attention(mx, W, p, h, v_other, lam, dtype, sigmoid, portions_of, tiled, window=0):
     """The framework's side of one attention mixer without its projections' library products: bias / norm / blend / store,
     then the attention over the pool, for sequences fed in the given portions. -> per sequence [T, heads * vdim]."""
     from swiftllm_amd.model_config import RatilornAttentionConfig
     from swiftllm_amd.worker.kernels.sigmoid_attn import sigmoid_attention
     from swiftllm_amd.worker.kernels.window_attn import AttentionSpec, masked_attention, qkv_bias_norm_store
     mixer = RatilornAttentionConfig(mx, sigmoid=sigmoid)
+    mixer.window = window       # (an argument of the kernels; the design itself sees every earlier key)
     dev = lambda name: W[p + name].float().cuda().contiguous()
     wqkv = torch.cat((W[p + "q"], W[p + "k"], W[p + "v"]), dim=0)
     lens = [x.shape[0] for x in h]
@@ -263,8 +264,9 @@ def test_sigmoid_attention_on_the_matrix_core(H, G, d, e, lens, dtype):
     _check_attention(H, G, d, e, lens, dtype, True, True, sizes=((1000,), (7, 1, 2, 16, 1), (1,)), blend=True)
 
 
+@pytest.mark.parametrize("far", [13, 15, 16, 271, 272])      # inside a page, on both sides of a page border, near and far
 @pytest.mark.parametrize("dtype,tiled,d", [(torch.float32, False, 24), (torch.bfloat16, True, 64), (torch.bfloat16, False, 24)])
-def test_a_far_key_among_hundreds_is_found(dtype, tiled, d):
+def test_a_far_key_among_hundreds_is_found(dtype, tiled, d, far):
     """Every key but one is pushed far below the sigmoid's threshold; the one that stands out lies hundreds of positions back,
     beyond many page borders, and the distance term takes its full toll. Leaving it out would change the last rows entirely."""
     def tune(W, p):
@@ -274,7 +276,7 @@ def test_a_far_key_among_hundreds_is_found(dtype, tiled, d):
         for nm in ("q", "k"):
             W[p + nm].zero_()
             W[p + nm + ".b"].zero_()
-    n, far = 420, 13
+    n = 420
     mx, W = _attention_weights(2, 1, d, 16, 24, 5, True)
     p = "l0.mix."
     tune(W, p)
@@ -300,6 +302,38 @@ def test_a_far_key_among_hundreds_is_found(dtype, tiled, d):
         got = _run_attention(mx, W, p, [h], None, 0.0, dtype, True, [cut(n, sizes)], tiled)[0]
         tol = 3e-5 if dtype == torch.float32 else 3e-2
         assert float((got[-3:].double() - want[-3:]).abs().max()) < tol * float(shown)
+
+
+@pytest.mark.parametrize("dtype,tiled,d,window", [(torch.float32, False, 24, 21), (torch.bfloat16, True, 64, 21),
+                                                  (torch.bfloat16, True, 32, 16), (torch.float32, False, 8, 1)])
+def test_sigmoid_attention_inside_a_window(dtype, tiled, d, window):
+    """The kernels' window argument: query i sees keys i - window + 1 .. i. Scores depend on positions through i - j only, so
+    the plain evaluation of the last `window` tokens alone gives query i's row. The key just inside the window and the one
+    just outside are made to stand out: one key more or less changes the row by several times the tolerance."""
+    n = 70
+    mx, W = _attention_weights(4, 2, d, 16, 24, 11, True)
+    p = "l0.mix."
+    W[p + "pb"].fill_(-6.0)
+    for nm in ("q", "k"):
+        W[p + nm].zero_()
+        W[p + nm + ".b"].zero_()
+    W[p + "q"][:, 0] = 8.0
+    W[p + "k"][:, 1] = 8.0
+    mx["scale"] = 12.0 / d
+    g = torch.Generator().manual_seed(4)
+    h = torch.randn(n, 24, generator=g).to(torch.bfloat16).float() * 0.1
+    h[:, :2] = 0
+    h[:, 0] = 1.0               # every query looks for the marked keys
+    h[::3, 1] = 1.0             # every third token is one: the window's edge passes over them
+    Wd = f64(W)
+    Wd[p + "o"] = torch.eye(4 * 16, dtype=torch.float64)
+    want = torch.stack([O.sigmoid_attention(h[max(0, i - window + 1):i + 1].double(), Wd, p, mx, EPS)[0][-1] for i in range(n)])
+    wider = torch.stack([O.sigmoid_attention(h[max(0, i - window):i + 1].double(), Wd, p, mx, EPS)[0][-1] for i in range(n)])
+    assert float((want - wider).abs().max()) > 0.1 * float(want.abs().max()), "the test's weights do not show the edge"
+    tol = 3e-5 if dtype == torch.float32 else 3e-2
+    for sizes in ((1000,), (33, 1), (5, 2, 16)):
+        got = _run_attention(mx, W, p, [h], None, 0.0, dtype, True, [cut(n, sizes)], tiled, window=window)[0]
+        assert float((got.double() - want).abs().max()) < tol * float(want.abs().max()), sizes
 
 
 @pytest.mark.parametrize("H,G,d,e,lens,dtype,tiled", [(4, 2, 16, 24, (150, 37), torch.float32, False),
@@ -514,9 +548,10 @@ def varied_config():
     the first attention layer, an attention layer that does not blend, a width that is no multiple of 8."""
     layers = [
         O.parallel_layer(heads=3, kv_heads=1, dim=24, vdim=8, s_heads=4, s_vdim=6, state=10, groups=2, conv=1, norm_groups=3,
+                         scale=0.31,
                          mlp=O.moe_mlp(ff=12, experts=6, top=1, groups=(6, 2), shared=0)),
-        O.attention_layer(heads=6, kv_heads=3, dim=16, vdim=8, v_mix=False, mlp=None),
-        O.attention_layer(heads=3, kv_heads=1, dim=24, vdim=24, v_mix=True, mlp=O.dense_mlp(36)),
+        O.attention_layer(heads=6, kv_heads=3, dim=16, vdim=8, v_mix=False, scale=0.4, mlp=None),
+        O.attention_layer(heads=3, kv_heads=1, dim=24, vdim=24, v_mix=True, scale=0.11, mlp=O.dense_mlp(36)),
         O.parallel_layer(heads=2, kv_heads=2, dim=8, vdim=40, s_heads=1, s_vdim=20, state=33, groups=1, conv=5, norm_groups=1,
                          mlp=O.moe_mlp(ff=8, experts=3, top=3, groups=None, shared=20)),
         O.attention_layer(heads=2, kv_heads=2, dim=32, vdim=12, v_mix=True, mlp=O.moe_mlp(ff=16, experts=9, top=2,
