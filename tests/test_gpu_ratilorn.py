@@ -255,7 +255,8 @@ def test_sigmoid_attention_fp32(H, G, d, e, lens):
 
 
 @pytest.mark.parametrize("H,G,d,e,lens", [(8, 4, 64, 32, (150, 37)), (4, 1, 64, 64, (70,)), (6, 3, 32, 32, (1, 2, 33)),
-                                          (16, 4, 128, 128, (64,)), (3, 3, 96, 96, (49,)), (20, 4, 48, 48, (40,))])
+                                          (16, 4, 128, 128, (64,)), (3, 3, 96, 96, (49,)), (20, 4, 48, 48, (40,)),
+                                          (32, 8, 128, 128, (40,))])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_sigmoid_attention_on_the_matrix_core(H, G, d, e, lens, dtype):
     from swiftllm_amd.model_config import RatilornAttentionConfig
@@ -345,7 +346,7 @@ def test_softmax_attention_with_biases_and_weighted_norm(H, G, d, e, lens, dtype
 
 @pytest.mark.parametrize("heads,P,N,groups,conv,parts,lens", [(3, 8, 12, 1, 3, 1, (70, 9)), (4, 24, 20, 2, 1, 2, (33,)),
                                                              (2, 32, 48, 2, 4, 1, (40, 1, 2)), (6, 16, 128, 3, 2, 3, (21,)),
-                                                             (1, 64, 16, 1, 5, 4, (50,))])
+                                                             (1, 64, 16, 1, 5, 4, (50,)), (2, 8, 256, 1, 2, 1, (37,))])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_state_space_mixer_in_portions_and_reused_slots(heads, P, N, groups, conv, parts, lens, dtype):
     from swiftllm_amd.model_config import StateSpaceConfig
