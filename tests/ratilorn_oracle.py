@@ -13,8 +13,6 @@ Notation: h [T, width] is a sublayer's input, W["name"] a checkpoint tensor, pos
                 in front and a gated grouped RMS norm behind
     ff:         down(silu(gate h) * up h), dense or as experts chosen by a sigmoid router with group-limited top-k
 """
-import math
-
 import torch
 
 

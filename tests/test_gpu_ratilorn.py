@@ -412,7 +412,6 @@ def test_sigmoid_router_with_group_limited_choice(experts, top, groups):
 @pytest.mark.parametrize("experts,top,groups,shared", [(8, 2, (4, 2), 16), (5, 1, None, 0), (6, 6, (3, 3), 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_mixture_of_gated_units(experts, top, groups, shared, n, dtype):
-    from swiftllm_amd.model_config import RatilornLayerConfig
     from swiftllm_amd.worker.layers.ratilorn_layer import RatilornFeedForward
     from swiftllm_amd.worker.ratilorn_weight import RatilornLayerWeight
     from swiftllm_amd.model_config import RatilornModelConfig

@@ -176,7 +176,6 @@ def test_layer_norms_the_result_not_the_input():
 
 
 def test_block_and_slot_layout():
-    from swiftllm_amd.engine_config import EngineConfig
     from swiftllm_amd.worker.ratilorn_model import RatilornModel
     cfg = O.make_config()
     mcfg = RatilornModelConfig(cfg)
