@@ -173,7 +173,8 @@ __global__ __launch_bounds__(kQkThreads) void qkv_bias_norm_store_kernel(
         // 16-bit heads of 32 / 64 / 128 elements on 16-byte-aligned rows: d / 8 lanes per head move 16 bytes each and several
         // heads share a wave (the group reduction stays inside d / 8 aligned lanes)
         wide = (d == 32 || d == 64 || d == 128) && (tok_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(qkv) & 15) == 0 &&
-               (!store || ((reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 && (block_stride & 7) == 0));
+               (!store || ((reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 && (block_stride & 7) == 0)) &&
+               ((reinterpret_cast<uintptr_t>(q_b) | reinterpret_cast<uintptr_t>(k_b)) & 15) == 0;
         if (wide) {
             const int lph = d >> 3;                 // lanes per head: 4, 8 or 16
             const int hpw = 64 / lph;               // heads per wave and pass
@@ -189,9 +190,17 @@ __global__ __launch_bounds__(kQkThreads) void qkv_bias_norm_store_kernel(
                 for (int j = 0; j < 8; ++j) v[j] = 0.f;
                 if (live) {
                     const vec8_t<T> x = load8(src);
-                    const float *bp = bias ? bias + static_cast<int64_t>(is_q ? h : h - H) * d + el * 8 : nullptr;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) v[j] = to_f(x[j]) + (bp ? bp[j] : 0.f);
+                    for (int j = 0; j < 8; ++j) v[j] = to_f(x[j]);
+                    if (bias) {     // (fp32 tensors start 16-byte aligned and h * d + 8 el is a multiple of 8)
+                        const float *bp = bias + static_cast<int64_t>(is_q ? h : h - H) * d + el * 8;
+                        const float4_t b0 = *reinterpret_cast<const float4_t *>(bp), b1 = *reinterpret_cast<const float4_t *>(bp + 4);
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            v[j] += b0[j];
+                            v[4 + j] += b1[j];
+                        }
+                    }
                 }
                 float ss = 0.f;
 #pragma unroll
@@ -230,6 +239,44 @@ __global__ __launch_bounds__(kQkThreads) void qkv_bias_norm_store_kernel(
     }
     T *vsrc = row + static_cast<int64_t>(H + G) * d;
     const T *vo = v_other ? v_other + t * v_other_stride : nullptr;
+    if constexpr (sizeof(T) == 2) {
+        // value heads whose size is a multiple of 8, on 16-byte-aligned rows: 8 columns per lane (the same sums as below)
+        const bool vwide = wide && (dv & 7) == 0 && ((static_cast<int64_t>(H + G) * d) & 7) == 0 &&
+                           (!v_b || (reinterpret_cast<uintptr_t>(v_b) & 15) == 0) &&
+                           (!vo || ((v_other_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(v_other) & 15) == 0));
+        if (vwide) {
+            for (int i = threadIdx.x * 8; i < G * dv; i += kQkThreads * 8) {
+                const vec8_t<T> x = load8(vsrc + i);
+                float v[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = to_f(x[j]);
+                if (v_b) {
+                    const float4_t b0 = *reinterpret_cast<const float4_t *>(v_b + i), b1 = *reinterpret_cast<const float4_t *>(v_b + i + 4);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        v[j] += b0[j];
+                        v[4 + j] += b1[j];
+                    }
+                }
+                if (vo) {
+                    const vec8_t<T> y = load8(vo + i);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) v[j] = (1.0f - mix) * v[j] + mix * to_f(y[j]);
+                }
+                vec8_t<T> o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = to_t<T>(v[j]);
+                store8(vsrc + i, o);
+                if (store) {
+                    const int g = i / dv, c = i - g * dv;       // (8 consecutive columns of one head)
+                    T *dst = v_cache + blk * block_stride + (static_cast<int64_t>(g) * dv + c) * kQkBlock + off;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) dst[j * kQkBlock] = o[j];       // transposed page
+                }
+            }
+            return;
+        }
+    }
     for (int i = threadIdx.x; i < G * dv; i += kQkThreads) {
         float v = to_f(vsrc[i]) + (v_b ? v_b[i] : 0.f);
         if (vo) v = (1.0f - mix) * v + mix * to_f(vo[i]);
